@@ -1,0 +1,152 @@
+/* mintccl.h - C ABI of libmintccl.so, the MI355X (gfx950) data path.
+ *
+ * The reference (huangs0/mintccl) has no FFI: its Python host functions launch
+ * Triton-JIT kernels directly, passing raw 64-bit device addresses with 0
+ * meaning "absent" (common.py:71), a byte count and rank/world integers.  Each
+ * entry point below names the reference launch it stands for.  A Python caller
+ * binds them with ctypes (see mintccl_amd/_lib.py).
+ *
+ * Conventions
+ *  - plain C types only; device addresses are void* / uint64_t, 0 = absent;
+ *  - every function returns 0 on success or a negative mint_error; none throws;
+ *  - all work is enqueued on the hipStream_t passed as void* (NULL = the
+ *    default stream); no call synchronises with the host;
+ *  - the caller owns every buffer and keeps it alive until the stream drains;
+ *  - the library keeps no per-call state: calls on different streams are
+ *    independent as long as their buffers are.
+ */
+#ifndef MINTCCL_H
+#define MINTCCL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MINT_MAX_RANKS 8
+#define MINT_LINE_BYTES 128u     /* protocol.py:47 BYTES_LL128_MSG */
+#define MINT_LINE_PAYLOAD 120u   /* protocol.py:48 BYTES_LL128_RAW */
+#define MINT_BLOCK_LINES 8u      /* lines one 64-lane access carries */
+#define MINT_BLOCK_MSG 1024u
+#define MINT_BLOCK_RAW 960u
+
+typedef enum {
+    MINT_OK = 0,
+    MINT_ERR_ARG = -1,        /* bad argument (null, range, unknown enum) */
+    MINT_ERR_ALIGN = -2,      /* address or stride not 16-byte aligned */
+    MINT_ERR_GEOMETRY = -3,   /* slot / wave geometry does not divide */
+    MINT_ERR_RESIDENCY = -4,  /* grid would not be co-resident on the device */
+    MINT_ERR_HIP = -5,        /* a HIP runtime call failed */
+    MINT_ERR_TOO_LARGE = -6   /* a row does not fit a 32-bit offset window */
+} mint_error;
+
+typedef enum { MINT_LAYOUT_PAIR = 0, MINT_LAYOUT_WAVE64 = 1 } mint_layout;
+typedef enum { MINT_F16 = 0, MINT_BF16 = 1, MINT_F32 = 2, MINT_BYTES = 3 } mint_dtype;
+typedef enum { MINT_PROTO_LL128 = 0, MINT_PROTO_SIMPLE = 1 } mint_protocol;
+typedef enum {
+    MINT_OP_SENDRECV = 0,      /* 2_sendrecv_indirect.py:44-93, 3_sendrecv_buffer.py:23-74 */
+    MINT_OP_BROADCAST = 1,     /* 4_broadcast.py:27-76 */
+    MINT_OP_REDUCE = 2,        /* 5_reduce.py:36-95 */
+    MINT_OP_ALLGATHER = 3,     /* 6_allgather.py:79-138 (spatial variant) */
+    MINT_OP_REDUCESCATTER = 4  /* 7_reducescatter.py:13-79 */
+} mint_op;
+typedef enum {
+    MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
+    MINT_PLACE_LOCAL = 1    /* every hop of a channel on the same XCD */
+} mint_placement;
+
+/* Status block written by the ring kernel (device memory, 4 x uint64, zeroed
+ * by the caller before launch).  word 0: 0 = OK, else 1 = a bounded wait ran
+ * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
+ * that gave up; word 2: step it waited for; word 3: abort flag polled by all
+ * other waits.  The reference has no abort path (common.py:106 is unused). */
+#define MINT_STATUS_WORDS 4
+
+/* One ring collective over `world` virtual ranks of one GPU.  It stands for the
+ * argument lists (recvbuff, sendbuff, inputbuff, outputbuff, count[, rank,
+ * dest, world_size, root]) of the reference kernels, for all ranks at once. */
+typedef struct {
+    int32_t op;            /* mint_op */
+    int32_t protocol;      /* mint_protocol */
+    int32_t dtype;         /* mint_dtype; MINT_BYTES for the copying ops */
+    int32_t world;         /* number of virtual ranks, 1..MINT_MAX_RANKS */
+    int32_t ring[MINT_MAX_RANKS + 1]; /* rank sequence, ring[world] == ring[0]
+                              (topology.py:56-93); for SENDRECV the route
+                              src..dst of route_len ranks */
+    int32_t route_len;     /* SENDRECV only: number of ranks on the route */
+    int32_t root;          /* BROADCAST / REDUCE root rank */
+    uint64_t input[MINT_MAX_RANKS];   /* per rank; 0 = absent */
+    uint64_t output[MINT_MAX_RANKS];  /* per rank; 0 = absent */
+    uint64_t staging[MINT_MAX_RANKS]; /* per rank, mint_ring_staging_bytes() each */
+    uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE: bytes of the buffer;
+                              ALLGATHER/REDUCESCATTER: bytes of one row */
+    uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER: bytes between rows */
+    uint32_t slot_bytes;   /* staging bytes of one step over all channels */
+    uint32_t nslots;       /* slots in the circular staging buffer */
+    uint32_t waves_per_channel_group; /* wave-channels per (pipeline, hop) */
+    uint32_t threads_per_block;       /* multiple of 64 */
+    int32_t placement;     /* mint_placement */
+    int32_t cache_policy;  /* 0 agent scope (sc1), 1 system scope (sc0 sc1) */
+    uint32_t flag_epoch;   /* must differ from every earlier launch that used
+                              the same staging memory; never 0 */
+    uint32_t spin_budget;  /* polls before a wait gives up; 0 = default */
+    uint64_t status;       /* device address of MINT_STATUS_WORDS uint64 */
+    uint32_t debug_skip_origin; /* testing: origin hop sends nothing */
+    uint32_t reserved;
+} mint_ring_op;
+
+int mint_version(void);
+const char* mint_strerror(int err);
+
+/* Compute units, XCDs and wavefront size of the current device. */
+int mint_device_info(int* compute_units, int* xcds, int* wave_size);
+
+/* XCC_ID of the XCD each of `blocks` thread blocks of a 1-D launch lands on
+ * (device uint32[blocks]); documents the block -> XCD dealing order that the
+ * placement option relies on. */
+int mint_xcd_map(int blocks, void* out, void* stream);
+
+/* Simple-protocol copy, 16 bytes per lane, persistent grid.
+ * Stands for recv_kernel (1_sendrecv_direct.py:31-54); also the HBM
+ * copy-bandwidth yardstick.  blocks = 0 picks a device-filling grid. */
+int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int threads,
+                     void* stream);
+
+/* Standalone LL128 codec (load_ll128 + send_ll128 / recv_ll128 + save_ll128,
+ * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride.
+ * msg must hold mint_ll128_packed_bytes(nbytes, layout).  bad_flags (device
+ * uint64, may be 0) is incremented once per line whose flag is not the
+ * expected one. */
+size_t mint_ll128_packed_bytes(size_t nbytes, int layout);
+int mint_ll128_pack(const void* raw, void* msg, size_t nbytes, uint64_t flag_base,
+                    uint64_t flag_stride, int layout, void* stream);
+int mint_ll128_unpack(const void* msg, void* raw, size_t nbytes, uint64_t flag_base,
+                      uint64_t flag_stride, int layout, void* bad_flags, void* stream);
+
+/* out = rn(a + b) elementwise with the reduction's own device function
+ * (SumFP16, primitive.py:232-247; comp_ll128, protocol.py:142-156). */
+int mint_elementwise_sum(const void* a, const void* b, void* out, size_t nelem, int dtype,
+                         void* stream);
+
+/* Bytes of staging each rank needs for this op (slots plus credit words). */
+size_t mint_ring_staging_bytes(const mint_ring_op* op);
+/* Blocks the launch will use; negative mint_error if the geometry is bad. */
+int mint_ring_grid_blocks(const mint_ring_op* op);
+/* Validate and enqueue one fused launch that runs every rank's kernel. */
+int mint_ring_launch(const mint_ring_op* op, void* stream);
+
+/* Torn-line probe: `pairs` producer wavefronts each rewrite one 1 KiB block
+ * `iters` times with lines whose payload is a function of the flag; the
+ * paired consumer wavefronts poll until the flag appears and count lines
+ * whose payload does not belong to the flag.  counters: device uint64[4] =
+ * {lines checked, torn lines, polls, timeouts}. */
+int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,
+                         int cache_policy, int placement, uint32_t flag_epoch,
+                         uint32_t spin_budget, void* counters, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINTCCL_H */

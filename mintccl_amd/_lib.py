@@ -1,0 +1,119 @@
+"""ctypes binding of ``libmintccl.so`` (C ABI declared in ``include/mintccl.h``).
+
+The shared library is the product's only compute path: if it is missing the
+import of any operator fails with an error that says how to build it.  There is
+no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_PKG)
+SO_PATH = os.path.join(_PKG, "libmintccl.so")
+SRC = os.path.join(_PKG, "csrc", "mintccl.hip")
+
+MAX_RANKS = 8
+STATUS_WORDS = 4
+
+OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6
+LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
+F16, BF16, F32, BYTES = 0, 1, 2, 3
+PROTO_LL128, PROTO_SIMPLE = 0, 1
+OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER = range(5)
+PLACE_SPREAD, PLACE_LOCAL = 0, 1
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed FP32 instructions are kept out of all device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+class RingOp(ctypes.Structure):
+    """``mint_ring_op`` of include/mintccl.h, field for field."""
+    _fields_ = [
+        ("op", ctypes.c_int32), ("protocol", ctypes.c_int32),
+        ("dtype", ctypes.c_int32), ("world", ctypes.c_int32),
+        ("ring", ctypes.c_int32 * (MAX_RANKS + 1)),
+        ("route_len", ctypes.c_int32), ("root", ctypes.c_int32),
+        ("input", ctypes.c_uint64 * MAX_RANKS),
+        ("output", ctypes.c_uint64 * MAX_RANKS),
+        ("staging", ctypes.c_uint64 * MAX_RANKS),
+        ("count_bytes", ctypes.c_uint64), ("row_stride", ctypes.c_uint64),
+        ("slot_bytes", ctypes.c_uint32), ("nslots", ctypes.c_uint32),
+        ("waves_per_channel_group", ctypes.c_uint32),
+        ("threads_per_block", ctypes.c_uint32),
+        ("placement", ctypes.c_int32), ("cache_policy", ctypes.c_int32),
+        ("flag_epoch", ctypes.c_uint32), ("spin_budget", ctypes.c_uint32),
+        ("status", ctypes.c_uint64),
+        ("debug_skip_origin", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/mintccl.h declares
+_vp, _sz, _u64, _u32, _i = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
+                            ctypes.c_uint32, ctypes.c_int)
+_ip = ctypes.POINTER(ctypes.c_int)
+_opp = ctypes.POINTER(RingOp)
+SYMBOLS = {
+    "mint_version": (_i, []),
+    "mint_strerror": (ctypes.c_char_p, [_i]),
+    "mint_device_info": (_i, [_ip, _ip, _ip]),
+    "mint_xcd_map": (_i, [_i, _vp, _vp]),
+    "mint_copy_simple": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
+    "mint_ll128_packed_bytes": (_sz, [_sz, _i]),
+    "mint_ll128_pack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp]),
+    "mint_ll128_unpack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp, _vp]),
+    "mint_elementwise_sum": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
+    "mint_ring_staging_bytes": (_sz, [_opp]),
+    "mint_ring_grid_blocks": (_i, [_opp]),
+    "mint_ring_launch": (_i, [_opp, _vp]),
+    "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
+}
+
+_lib = None
+
+
+def build(verbose: bool = False) -> str:
+    """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree)."""
+    cmd = ["hipcc", *HIPCC_FLAGS, "-o", SO_PATH, SRC]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed:\n{proc.stderr}")
+    if verbose:
+        print(" ".join(cmd))
+    return SO_PATH
+
+
+class MintError(RuntimeError):
+    def __init__(self, code: int, where: str):
+        self.code = code
+        msg = lib().mint_strerror(code).decode() if _lib is not None else str(code)
+        super().__init__(f"{where}: {msg} ({code})")
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            raise RuntimeError(
+                f"{SO_PATH} is missing: the HIP extension has not been built. "
+                "Run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(or mintccl_amd._lib.build()) in the repository root. "
+                "There is no CPU fallback.")
+        L = ctypes.CDLL(SO_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def check(code: int, where: str) -> None:
+    if code != OK:
+        raise MintError(code, where)

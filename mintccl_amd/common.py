@@ -1,0 +1,288 @@
+"""Configuration and the virtual-rank communicator.
+
+Mirrors the reference's ``common.py``: the tuning knobs keep their
+``MINTCCL_*`` names and defaults (``common.py:85-118``) but are read when an
+operator runs, not at import.  ``set_gpu`` / ``send_ptr`` / ``recv_ptr``
+(``common.py:10-38``) keep their names; with every rank living in one process
+on one GPU they reduce to a device choice and a pointer mailbox.
+"""
+from __future__ import annotations
+
+import contextlib
+import os
+import threading
+import time
+
+import torch
+
+from . import _lib
+
+NULL = 0                       # common.py:71
+WARP_SIZE = 64                 # common.py:104 is 32; a CDNA4 wavefront has 64 lanes
+VECTORIZED_BYTES = 16          # common.py:105
+SPINS_BEFORE_ABORT = 4000000   # common.py:106 (unused there, enforced here)
+
+
+def _env_int(name: str, default: int) -> int:
+    v = os.getenv(name)
+    return int(v) if v not in (None, "") else default
+
+
+def num_blocks() -> int:        # common.py:85
+    return _env_int("MINTCCL_NUM_BLOCKS", 16)
+
+
+def num_warps() -> int:         # common.py:92 (32-lane warps; two make a wavefront)
+    return _env_int("MINTCCL_NUM_WARPS", 16)
+
+
+def buff_size() -> int:         # common.py:101
+    return _env_int("MINTCCL_BUFFSIZE", 4194304)
+
+
+def num_slots() -> int:
+    return _env_int("MINTCCL_NSLOTS", 8)
+
+
+def world_size_env() -> int:
+    return _env_int("MINTCCL_WORLD_SIZE", 8)
+
+
+def protocol_env() -> int:
+    return {"ll128": _lib.PROTO_LL128, "simple": _lib.PROTO_SIMPLE}[
+        os.getenv("MINTCCL_PROTOCOL", "ll128").lower()]
+
+
+def placement_env() -> int:
+    return {"spread": _lib.PLACE_SPREAD, "local": _lib.PLACE_LOCAL}[
+        os.getenv("MINTCCL_PLACEMENT", "spread").lower()]
+
+
+def test_mode() -> bool:        # common.py:113 (any non-empty string enables it)
+    return bool(os.getenv("MINTCCL_TEST_MODE", ""))
+
+
+def test_count() -> int:        # common.py:115
+    return _env_int("MINTCCL_TEST_COUNT", 67108864)
+
+
+def verbose() -> bool:          # common.py:118
+    return bool(os.getenv("MINTCCL_TEST_VERBOSE", ""))
+
+
+DTYPE_CODE = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+
+
+class Timer:
+    """CPU / device timer context manager (``common.py:41-67``)."""
+
+    def __init__(self, device: bool = False, rank: int | None = None) -> None:
+        self.rank, self.device, self.elapsed = rank, device, 0.0
+
+    def __enter__(self):
+        if self.device:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+        else:
+            self.start = time.perf_counter_ns()
+        return self
+
+    def __exit__(self, *exc):
+        if self.device:
+            self.end.record()
+            torch.cuda.synchronize()
+            self.elapsed = self.start.elapsed_time(self.end) / 1e3
+        else:
+            self.elapsed = (time.perf_counter_ns() - self.start) / 1e9
+        tag = f"rank: {self.rank} " if self.rank is not None else ""
+        print(f"# {tag}time: {self.elapsed}s")
+
+
+class RingTimeout(RuntimeError):
+    """A bounded wait inside the ring kernel ran out (status word 0 != 0)."""
+
+
+def _largest_divisor_at_most(n: int, cap: int) -> int:
+    cap = max(1, min(n, cap))
+    for d in range(cap, 0, -1):
+        if n % d == 0:
+            return d
+    return 1
+
+
+class VirtualComm:
+    """N virtual ranks on one GPU: stands in for ``MPI.COMM_WORLD``.
+
+    Every rank owns a disjoint region of one staging allocation
+    (``nslots`` slots of ``buff_size / nslots`` bytes plus its credit words).
+    Ranks enter with ``with comm.rank(r):`` and call the reference-named
+    operators; the call that completes the set of participants enqueues ONE
+    fused launch that runs all ranks' kernels.
+    """
+
+    def __init__(self, world_size: int | None = None, device: str | torch.device = "cuda:0",
+                 buff_size_: int | None = None, nslots: int | None = None,
+                 protocol: int | None = None, placement: int | None = None,
+                 waves_per_rank: int | None = None, threads_per_block: int | None = None,
+                 cache_policy: int = 0, spin_budget: int = 0) -> None:
+        self.world_size = world_size if world_size is not None else world_size_env()
+        if not 1 <= self.world_size <= _lib.MAX_RANKS:
+            raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
+        self.device = torch.device(device)
+        self.buff_size = buff_size_ if buff_size_ is not None else buff_size()
+        self.nslots = nslots if nslots is not None else num_slots()
+        if self.buff_size % self.nslots:
+            raise ValueError("MINTCCL_BUFFSIZE must be a multiple of MINTCCL_NSLOTS")
+        self.slot_bytes = self.buff_size // self.nslots
+        self.protocol = protocol if protocol is not None else protocol_env()
+        self.placement = placement if placement is not None else placement_env()
+        # reference geometry: NUM_BLOCKS blocks of NUM_WARPS 32-lane warps per rank
+        self.waves_per_rank = (waves_per_rank if waves_per_rank is not None
+                               else max(1, num_blocks() * num_warps() // 2))
+        self.threads_per_block = (threads_per_block if threads_per_block is not None
+                                  else _env_int("MINTCCL_THREADS", 256))
+        self.cache_policy = cache_policy
+        self.spin_budget = spin_budget
+        self._lib = _lib.lib()          # fails loudly if the extension is missing
+        # slots + credit words (never more than slot_bytes / 4), zeroed: flag 0
+        # and credit 0 mean "nothing yet" (2_sendrecv_indirect.py:59-60).
+        self.rank_stride = self.buff_size + max(4096, self.slot_bytes // 4)
+        self.rank_stride = (self.rank_stride + 255) // 256 * 256
+        self.staging = torch.zeros(self.world_size * self.rank_stride, dtype=torch.uint8,
+                                   device=self.device)
+        self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int64, device=self.device)
+        self.epoch = 0
+        self._tls = threading.local()
+        self._pending: dict = {}
+        self._mailbox: dict = {}
+        self.last_grid = 0
+
+    # ---- MPI-like surface -------------------------------------------------
+    def Get_size(self) -> int:
+        return self.world_size
+
+    def Get_rank(self) -> int:
+        r = getattr(self._tls, "rank", None)
+        if r is None:
+            raise RuntimeError("no current rank: use `with comm.rank(r):`")
+        return r
+
+    @contextlib.contextmanager
+    def rank(self, r: int):
+        if not 0 <= r < self.world_size:
+            raise ValueError(f"rank {r} outside world of {self.world_size}")
+        prev = getattr(self._tls, "rank", None)
+        self._tls.rank = r
+        try:
+            yield self
+        finally:
+            self._tls.rank = prev
+
+    def run(self, fn) -> None:
+        """SPMD helper: ``fn(rank)`` for every rank in turn (like mpirun)."""
+        for r in range(self.world_size):
+            with self.rank(r):
+                fn(r)
+
+    def staging_ptr(self, r: int) -> int:
+        return self.staging.data_ptr() + r * self.rank_stride
+
+    # pointer mailbox (send_ptr / recv_ptr, common.py:22-38)
+    def send_ptr(self, ptr: int, peer: int) -> None:
+        self._mailbox.setdefault((self.Get_rank(), peer), []).append(ptr)
+
+    def recv_ptr(self, peer: int) -> int:
+        return self._mailbox[(peer, self.Get_rank())].pop(0)
+
+    # ---- collective registration -------------------------------------------
+    def post(self, key: str, needed: set, info) -> dict | None:
+        """Record this rank's arguments; return all of them once the ranks in
+        ``needed`` have posted."""
+        slot = self._pending.setdefault(key, {})
+        r = self.Get_rank()
+        if r in slot:
+            raise RuntimeError(f"rank {r} called {key} twice before the others joined")
+        slot[r] = info
+        if set(slot) >= needed:
+            del self._pending[key]
+            return slot
+        return None
+
+    # ---- launch -------------------------------------------------------------
+    def make_op(self, op: int, dtype: int, count_bytes: int, inputs: dict, outputs: dict,
+                ring: list[int], root: int = 0, row_stride: int = 0, route_len: int = 0,
+                protocol: int | None = None, skip_origin: bool = False) -> _lib.RingOp:
+        d = _lib.RingOp()
+        d.op, d.dtype, d.world = op, dtype, self.world_size
+        d.protocol = self.protocol if protocol is None else protocol
+        for i, r in enumerate(ring):
+            d.ring[i] = r
+        d.route_len, d.root = route_len, root
+        for r in range(self.world_size):
+            d.input[r] = inputs.get(r, NULL)
+            d.output[r] = outputs.get(r, NULL)
+            d.staging[r] = self.staging_ptr(r)
+        d.count_bytes, d.row_stride = count_bytes, row_stride
+        d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
+        pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER) else 1
+        if self.slot_bytes % (pipes * 1024):
+            raise ValueError("slot size must be a multiple of pipelines x 1 KiB")
+        step_blocks = self.slot_bytes // pipes // 1024
+        d.waves_per_channel_group = _largest_divisor_at_most(
+            step_blocks, max(1, self.waves_per_rank // pipes))
+        d.threads_per_block = self.threads_per_block
+        d.placement, d.cache_policy = self.placement, self.cache_policy
+        d.spin_budget = self.spin_budget
+        d.status = self.status.data_ptr()
+        d.debug_skip_origin = int(skip_origin)
+        return d
+
+    def launch(self, d: _lib.RingOp) -> None:
+        """Enqueue on the current stream; never synchronises."""
+        self.epoch += 1
+        d.flag_epoch = self.epoch
+        self.last_grid = self._lib.mint_ring_grid_blocks(d)
+        with torch.cuda.device(self.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            _lib.check(self._lib.mint_ring_launch(d, stream), "mint_ring_launch")
+
+    def check(self) -> None:
+        """Synchronise and raise ``RingTimeout`` if a wait gave up."""
+        torch.cuda.synchronize(self.device)
+        st = self.status.cpu().tolist()
+        if st[0] != 0:
+            self.status.zero_()
+            who = st[1]
+            raise RingTimeout(
+                f"ring kernel wait ran out: pipeline {who >> 32}, position "
+                f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]}")
+
+
+_default_comm: VirtualComm | None = None
+
+
+def get_comm() -> VirtualComm:
+    """The process-wide communicator (created on first use from the env)."""
+    global _default_comm
+    if _default_comm is None:
+        _default_comm = VirtualComm()
+    return _default_comm
+
+
+def set_comm(comm: VirtualComm | None) -> None:
+    global _default_comm
+    _default_comm = comm
+
+
+def set_gpu(rank: int) -> None:
+    """``common.py:10-17``: every virtual rank lives on the one visible GPU."""
+    torch.set_default_device("cuda:0")
+
+
+def send_ptr(ptr: int, peer: int) -> None:
+    get_comm().send_ptr(ptr, peer)
+
+
+def recv_ptr(peer: int) -> int:
+    return get_comm().recv_ptr(peer)

@@ -1,0 +1,211 @@
+// Stand-alone kernels: simple-protocol copy, LL128 codec, element sum,
+// torn-line probe, block -> XCD map.
+#pragma once
+#include "protocol.hpp"
+
+namespace mint {
+
+// recv_kernel (1_sendrecv_direct.py:31-54): persistent grid-stride copy,
+// 16 bytes per lane, four independent accesses in flight per lane.
+__global__ void __launch_bounds__(1024) copy_simple_kernel(const uint8_t* __restrict__ src,
+                                                           uint8_t* __restrict__ dst,
+                                                           uint64_t nbytes) {
+    const uint64_t nvec = nbytes >> 4;
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
+    uint64_t i = tid;
+    for (; i + 3 * nthr < nvec; i += 4 * nthr) {
+        u32x4 a = ld128_stream(src + (i << 4));
+        u32x4 b = ld128_stream(src + ((i + nthr) << 4));
+        u32x4 c = ld128_stream(src + ((i + 2 * nthr) << 4));
+        u32x4 d = ld128_stream(src + ((i + 3 * nthr) << 4));
+        st128_stream(dst + (i << 4), a);
+        st128_stream(dst + ((i + nthr) << 4), b);
+        st128_stream(dst + ((i + 2 * nthr) << 4), c);
+        st128_stream(dst + ((i + 3 * nthr) << 4), d);
+    }
+    for (; i < nvec; i += nthr) st128_stream(dst + (i << 4), ld128_stream(src + (i << 4)));
+    if (tid < (nbytes & 15u)) dst[(nvec << 4) + tid] = src[(nvec << 4) + tid];
+}
+
+// ---- LL128 codec, wave64 layout: one wavefront per block -------------------
+__global__ void __launch_bounds__(256) pack_wave64_kernel(const uint8_t* __restrict__ raw,
+                                                          uint8_t* __restrict__ msg,
+                                                          uint64_t nbytes, uint32_t nblocks,
+                                                          uint64_t flag_base, uint64_t flag_stride) {
+    const LaneMap m;
+    const uint32_t waves = gridDim.x * (blockDim.x >> 6);
+    const uint32_t wave = blockIdx.x * (blockDim.x >> 6) + (uint32_t)wave_in_block();
+    for (uint32_t g = wave; g < nblocks; g += waves) {
+        u32x4 v = ll_load_raw(raw, nbytes, g, m);
+        const uint64_t flag = flag_base + ((uint64_t)g * 8u + m.line) * flag_stride;
+        if (m.flag_lane) { v.z = (uint32_t)flag; v.w = (uint32_t)(flag >> 32); }
+        *reinterpret_cast<u32x4*>(msg + (uint64_t)g * kBlockMsg + m.lane * 16u) = v;
+    }
+}
+__global__ void __launch_bounds__(256) unpack_wave64_kernel(const uint8_t* __restrict__ msg,
+                                                            uint8_t* __restrict__ raw,
+                                                            uint64_t nbytes, uint32_t nblocks,
+                                                            uint64_t flag_base,
+                                                            uint64_t flag_stride,
+                                                            unsigned long long* bad_flags) {
+    const LaneMap m;
+    const uint32_t waves = gridDim.x * (blockDim.x >> 6);
+    const uint32_t wave = blockIdx.x * (blockDim.x >> 6) + (uint32_t)wave_in_block();
+    uint32_t bad = 0;
+    for (uint32_t g = wave; g < nblocks; g += waves) {
+        u32x4 v = *reinterpret_cast<const u32x4*>(msg + (uint64_t)g * kBlockMsg + m.lane * 16u);
+        const uint64_t flag = flag_base + ((uint64_t)g * 8u + m.line) * flag_stride;
+        if (m.flag_lane && (v.z != (uint32_t)flag || v.w != (uint32_t)(flag >> 32))) ++bad;
+        ll_save_raw(raw, nbytes, g, m, v);
+    }
+    if (bad && bad_flags) atomicAdd(bad_flags, (unsigned long long)bad);
+}
+
+// ---- LL128 codec, reference pair layout: one thread per 16-byte message
+// lane, 8 threads per line, exactly the reference's lane roles
+// (protocol.py:57-100,132-137).
+__device__ __forceinline__ void pair_lane(uint64_t t, uint64_t& line, uint32_t& k,
+                                          uint64_t& raw_off, uint32_t& raw_len) {
+    line = t >> 3;
+    k = (uint32_t)(t & 7u);
+    const uint64_t pair_base = (line >> 1) * 240u;
+    const bool second = line & 1u;
+    if (k != 7u) { raw_off = pair_base + (second ? 128u : 0u) + k * 16u; raw_len = 16u; }
+    else         { raw_off = pair_base + (second ? 120u : 112u);         raw_len = 8u; }
+}
+__global__ void __launch_bounds__(256) pack_pair_kernel(const uint8_t* __restrict__ raw,
+                                                        uint8_t* __restrict__ msg,
+                                                        uint64_t nbytes, uint64_t nlines,
+                                                        uint64_t flag_base, uint64_t flag_stride) {
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < nlines * 8u; t += nthr) {
+        uint64_t line, raw_off; uint32_t k, raw_len;
+        pair_lane(t, line, k, raw_off, raw_len);
+        u32x4 v = load_guarded(raw, raw_off, raw_len, nbytes);
+        if (k == 7u) {
+            const uint64_t flag = flag_base + line * flag_stride;
+            v.z = (uint32_t)flag; v.w = (uint32_t)(flag >> 32);
+        }
+        *reinterpret_cast<u32x4*>(msg + (t << 4)) = v;
+    }
+}
+__global__ void __launch_bounds__(256) unpack_pair_kernel(const uint8_t* __restrict__ msg,
+                                                          uint8_t* __restrict__ raw,
+                                                          uint64_t nbytes, uint64_t nlines,
+                                                          uint64_t flag_base, uint64_t flag_stride,
+                                                          unsigned long long* bad_flags) {
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
+    uint32_t bad = 0;
+    for (uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; t < nlines * 8u; t += nthr) {
+        uint64_t line, raw_off; uint32_t k, raw_len;
+        pair_lane(t, line, k, raw_off, raw_len);
+        u32x4 v = *reinterpret_cast<const u32x4*>(msg + (t << 4));
+        if (k == 7u) {
+            const uint64_t flag = flag_base + line * flag_stride;
+            if (v.z != (uint32_t)flag || v.w != (uint32_t)(flag >> 32)) ++bad;
+        }
+        store_guarded(raw, raw_off, raw_len, nbytes, v);
+    }
+    if (bad && bad_flags) atomicAdd(bad_flags, (unsigned long long)bad);
+}
+
+// ---- out = rn(a + b) ------------------------------------------------------
+template <int DT>
+__global__ void __launch_bounds__(256) sum_kernel(const uint8_t* __restrict__ a,
+                                                  const uint8_t* __restrict__ b,
+                                                  uint8_t* __restrict__ out, uint64_t nbytes) {
+    const uint64_t nvec = nbytes >> 4;
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = tid; i < nvec; i += nthr) {
+        u32x4 x = *reinterpret_cast<const u32x4*>(a + (i << 4));
+        u32x4 y = *reinterpret_cast<const u32x4*>(b + (i << 4));
+        *reinterpret_cast<u32x4*>(out + (i << 4)) = add_rn<DT>(x, y);
+    }
+    if (tid == 0 && (nbytes & 15u)) {
+        u32x4 x = load_guarded(a, nvec << 4, 16u, nbytes);
+        u32x4 y = load_guarded(b, nvec << 4, 16u, nbytes);
+        store_guarded(out, nvec << 4, 16u, nbytes, add_rn<DT>(x, y));
+    }
+}
+
+// ---- block -> XCD map -------------------------------------------------------
+__global__ void xcd_map_kernel(uint32_t* out) {
+    if (threadIdx.x == 0) out[blockIdx.x] = (uint32_t)xcc_id();
+}
+
+// ---- torn-line probe --------------------------------------------------------
+// The payload of a line is a function of its flag, so a consumer that sees
+// the flag can tell whether the other 120 bytes belong to it.
+__device__ __forceinline__ uint32_t probe_word(uint32_t flag_lo, uint32_t lane, uint32_t d) {
+    return (flag_lo * 2654435761u) ^ (lane * 0x9E3779B1u + d * 0x85EBCA77u + 0x1234567u);
+}
+constexpr uint32_t kProbeDepth = 4;   // blocks per pair, reused round-robin
+
+template <int CP>
+__global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint32_t pairs,
+                                                         uint32_t iters, int placement,
+                                                         uint32_t epoch, uint32_t budget,
+                                                         unsigned long long* counters) {
+    const LaneMap m;
+    const uint32_t wpb = blockDim.x >> 6;
+    const uint32_t pair_blocks = (pairs + wpb - 1) / wpb;
+    uint32_t pb; bool producer;
+    if (placement == 1) { pb = blockIdx.x % pair_blocks; producer = blockIdx.x < pair_blocks; }
+    else                { pb = blockIdx.x >> 1;          producer = !(blockIdx.x & 1u); }
+    const uint32_t pair = pb * wpb + (uint32_t)wave_in_block();
+    if (pair >= pairs) return;
+    const uint32_t data_bytes = pairs * kProbeDepth * kBlockMsg;
+    const Window win(staging, data_bytes);
+    uint64_t* tail = reinterpret_cast<uint64_t*>(staging + data_bytes + (uint64_t)pair * 128u);
+    const uint64_t flag_hi = (uint64_t)epoch << 32;
+    unsigned long long checked = 0, torn = 0, polls = 0, timeouts = 0;
+    uint32_t seen = 0;
+    for (uint32_t t = 0; t < iters; ++t) {
+        const uint32_t off = (pair * kProbeDepth + t % kProbeDepth) * kBlockMsg;
+        const uint64_t flag = flag_hi | ((uint64_t)t * 8u + m.line + 1u);
+        const uint32_t flo = (uint32_t)flag;
+        if (producer) {
+            if (t >= kProbeDepth) {
+                bool ok = false;
+                for (uint32_t spins = 0; spins <= budget; ++spins) {
+                    uint64_t v = ld64_agent(tail);
+                    uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+                    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+                    if (hi == epoch && lo >= t - kProbeDepth + 1) { ok = true; seen = lo; break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                if (!ok) { ++timeouts; break; }
+            }
+            u32x4 v = {probe_word(flo, m.lane, 0), probe_word(flo, m.lane, 1),
+                       probe_word(flo, m.lane, 2), probe_word(flo, m.lane, 3)};
+            ll_send<CP>(win, off, v, flag, m);
+        } else {
+            u32x4 v; bool ok = false;
+            for (uint32_t spins = 0; spins <= budget; ++spins) {
+                compiler_fence();
+                ++polls;
+                if (ll_poll<CP>(win, off, flag, m, v)) { ok = true; break; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (!ok) { ++timeouts; break; }
+            bool bad = v.x != probe_word(flo, m.lane, 0) || v.y != probe_word(flo, m.lane, 1);
+            if (!m.flag_lane)
+                bad = bad || v.z != probe_word(flo, m.lane, 2) || v.w != probe_word(flo, m.lane, 3);
+            const uint64_t mask = __ballot(bad);
+            for (uint32_t j = 0; j < 8u; ++j) torn += ((mask >> (8u * j)) & 0xFFull) ? 1u : 0u;
+            checked += 8u;
+            if (lane_id() == 0) st64_agent(tail, flag_hi | (uint64_t)(t + 1));
+        }
+    }
+    (void)seen;
+    if (lane_id() == 0) {
+        if (checked) atomicAdd(counters + 0, checked);
+        if (torn) atomicAdd(counters + 1, torn);
+        if (polls) atomicAdd(counters + 2, polls);
+        if (timeouts) atomicAdd(counters + 3, timeouts);
+    }
+}
+
+}  // namespace mint

@@ -1,0 +1,387 @@
+// libmintccl.so - C ABI over the HIP kernels (see include/mintccl.h).
+#include "../../include/mintccl.h"
+
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+#include "ring.hpp"
+
+using namespace mint;
+
+namespace {
+
+constexpr int kVersion = 100;   // 0.1.0
+constexpr uint32_t kDefaultSpinBudget = 4000000u;
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
+inline bool aligned16(const void* p) { return aligned16(reinterpret_cast<uint64_t>(p)); }
+
+int device_cus() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        return 0;
+    return cus;
+}
+
+int launch_status() { return hipGetLastError() == hipSuccess ? MINT_OK : MINT_ERR_HIP; }
+
+bool reducing(int op) { return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER; }
+
+// Everything the launch derives from the descriptor.
+struct Plan {
+    RingArgs args;
+    int blocks, threads, unroll;
+    bool empty;
+};
+
+int make_plan(const mint_ring_op* op, Plan* plan) {
+    if (!op || !plan) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_REDUCESCATTER) return MINT_ERR_ARG;
+    if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
+    if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
+    if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
+    if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
+    if (op->cache_policy != 0 && op->cache_policy != 1) return MINT_ERR_ARG;
+    if (op->placement != MINT_PLACE_SPREAD && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
+    if (op->flag_epoch == 0 || !op->status) return MINT_ERR_ARG;
+    if (op->threads_per_block == 0 || op->threads_per_block % 64 || op->threads_per_block > 512)
+        return MINT_ERR_ARG;
+    if (op->nslots == 0 || op->slot_bytes == 0) return MINT_ERR_GEOMETRY;
+    if ((uint64_t)op->nslots * op->slot_bytes >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
+
+    RingArgs& a = plan->args;
+    a = RingArgs{};
+    a.op = op->op;
+    a.world = op->world;
+    const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER;
+    a.pipes = rowwise ? op->world : 1;
+
+    // ring / route
+    bool seen[MINT_MAX_RANKS] = {};
+    if (op->op == MINT_OP_SENDRECV) {
+        if (op->route_len < 1 || op->route_len > op->world) return MINT_ERR_ARG;
+        a.cyc_len = op->route_len;
+    } else {
+        a.cyc_len = op->world;
+        if (op->ring[op->world] != op->ring[0]) return MINT_ERR_ARG;
+    }
+    for (int i = 0; i < a.cyc_len; ++i) {
+        int r = op->ring[i];
+        if (r < 0 || r >= op->world || seen[r]) return MINT_ERR_ARG;
+        seen[r] = true;
+        a.cyc[i] = (uint8_t)r;
+    }
+    auto index_of = [&](int rank) {
+        for (int i = 0; i < a.cyc_len; ++i) if (a.cyc[i] == rank) return i;
+        return -1;
+    };
+    switch (op->op) {
+        case MINT_OP_SENDRECV:  a.hops = a.cyc_len - 1; a.start[0] = 0; break;
+        case MINT_OP_BROADCAST:
+        case MINT_OP_REDUCE: {
+            if (op->root < 0 || op->root >= op->world) return MINT_ERR_ARG;
+            a.hops = op->op == MINT_OP_BROADCAST ? op->world - 1 : op->world;
+            a.start[0] = (uint8_t)index_of(op->root);
+            break;
+        }
+        default:
+            a.hops = op->op == MINT_OP_ALLGATHER ? op->world - 1 : op->world;
+            for (int p = 0; p < op->world; ++p) a.start[p] = (uint8_t)index_of(p);
+    }
+
+    a.row_bytes = op->count_bytes;
+    a.row_stride = rowwise ? op->row_stride : 0;
+    plan->empty = op->count_bytes == 0 || op->world == 1 ||
+                  (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);
+    if (rowwise && (op->row_stride < op->count_bytes || !aligned16(op->row_stride)))
+        return MINT_ERR_ALIGN;
+    const int dt_size = op->dtype == MINT_F32 ? 4 : (op->dtype == MINT_BYTES ? 1 : 2);
+    if (op->count_bytes % dt_size) return MINT_ERR_ARG;
+
+    // which ranks need which buffers
+    for (int p = 0; p < a.pipes && !plan->empty; ++p) {
+        for (int h = 0; h <= a.hops; ++h) {
+            const int rank = a.cyc[(a.start[p] + h) % a.cyc_len];
+            const bool origin = h == 0, sink = h == a.hops;
+            const bool load = origin || (reducing(op->op) && !sink);
+            const bool save = sink || ((op->op == MINT_OP_BROADCAST ||
+                                        op->op == MINT_OP_ALLGATHER) && !origin);
+            if (load && (!op->input[rank] || !aligned16(op->input[rank])))
+                return op->input[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+            if (save && (!op->output[rank] || !aligned16(op->output[rank])))
+                return op->output[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+            if (!origin && (!op->staging[rank] || !aligned16(op->staging[rank])))
+                return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+        }
+    }
+    for (int r = 0; r < op->world; ++r) {
+        a.input[r] = op->input[r];
+        a.output[r] = op->output[r];
+        a.staging[r] = op->staging[r];
+    }
+
+    // geometry
+    a.slot_bytes = op->slot_bytes;
+    a.nslots = op->nslots;
+    if (op->slot_bytes % ((uint32_t)a.pipes * kBlockMsg)) return MINT_ERR_GEOMETRY;
+    a.step_msg = op->slot_bytes / (uint32_t)a.pipes;
+    a.step_blocks = a.step_msg / kBlockMsg;
+    if (op->waves_per_channel_group == 0 || a.step_blocks % op->waves_per_channel_group)
+        return MINT_ERR_GEOMETRY;
+    a.waves = (int)op->waves_per_channel_group;
+    a.k_per_wave = a.step_blocks / (uint32_t)a.waves;
+    const uint32_t raw_per_block = op->protocol == MINT_PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
+    const uint64_t nblocks = (op->count_bytes + raw_per_block - 1) / raw_per_block;
+    if (nblocks >= (1ull << 28)) return MINT_ERR_TOO_LARGE;
+    a.nblocks = (uint32_t)nblocks;
+    a.steps = (a.nblocks + a.step_blocks - 1) / a.step_blocks;
+    a.credit_off = a.nslots * a.slot_bytes;
+    a.epoch = op->flag_epoch;
+    a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
+    a.status = reinterpret_cast<uint64_t*>(op->status);
+    a.skip_origin = op->debug_skip_origin;
+    a.placement = op->placement;
+
+    const int waves_per_block = (int)op->threads_per_block / 64;
+    plan->threads = (int)op->threads_per_block;
+    if (a.waves < waves_per_block) plan->threads = a.waves * 64;
+    a.blocks_per_group = (a.waves * 64 + plan->threads - 1) / plan->threads;
+    plan->blocks = a.pipes * (a.hops + 1) * a.blocks_per_group;
+    plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
+    return MINT_OK;
+}
+
+template <int PROTO, int DT, int CP>
+int launch_ring_u(const Plan& plan, hipStream_t stream) {
+    void (*kernel)(const RingArgs) = nullptr;
+    switch (plan.unroll) {
+        case 4: kernel = ring_kernel<PROTO, DT, CP, 4>; break;
+        case 2: kernel = ring_kernel<PROTO, DT, CP, 2>; break;
+        default: kernel = ring_kernel<PROTO, DT, CP, 1>; break;
+    }
+    // Every wavefront of the launch polls words other wavefronts write, so
+    // the whole grid has to be resident at once.
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) != hipSuccess)
+        return MINT_ERR_HIP;
+    if (plan.blocks > per_cu * device_cus()) return MINT_ERR_RESIDENCY;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
+                       plan.args);
+    return launch_status();
+}
+template <int PROTO, int DT>
+int launch_ring_cp(const Plan& plan, int cache_policy, hipStream_t stream) {
+    return cache_policy == 0 ? launch_ring_u<PROTO, DT, CP_AGENT>(plan, stream)
+                             : launch_ring_u<PROTO, DT, CP_SYSTEM>(plan, stream);
+}
+template <int PROTO>
+int launch_ring_dt(const Plan& plan, int dtype, int cache_policy, hipStream_t stream) {
+    switch (dtype) {
+        case MINT_F16: return launch_ring_cp<PROTO, DT_F16>(plan, cache_policy, stream);
+        case MINT_BF16: return launch_ring_cp<PROTO, DT_BF16>(plan, cache_policy, stream);
+        case MINT_F32: return launch_ring_cp<PROTO, DT_F32>(plan, cache_policy, stream);
+        default: return launch_ring_cp<PROTO, DT_BYTES>(plan, cache_policy, stream);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mint_version(void) { return kVersion; }
+
+const char* mint_strerror(int err) {
+    switch (err) {
+        case MINT_OK: return "ok";
+        case MINT_ERR_ARG: return "bad argument";
+        case MINT_ERR_ALIGN: return "address or stride not 16-byte aligned";
+        case MINT_ERR_GEOMETRY: return "slot / wave geometry does not divide";
+        case MINT_ERR_RESIDENCY: return "grid would not be co-resident on the device";
+        case MINT_ERR_HIP: return "HIP runtime call failed";
+        case MINT_ERR_TOO_LARGE: return "size does not fit the kernel's 32-bit counters";
+        default: return "unknown error";
+    }
+}
+
+int mint_device_info(int* compute_units, int* xcds, int* wave_size) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MINT_ERR_HIP;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return MINT_ERR_HIP;
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (wave_size) *wave_size = prop.warpSize;
+    if (xcds) {
+        // Blocks are dealt round-robin over the XCDs: read the XCC_ID of the
+        // first 64 blocks and count the distinct values.
+        uint32_t* d = nullptr;
+        if (hipMalloc(&d, 64 * sizeof(uint32_t)) != hipSuccess) return MINT_ERR_HIP;
+        hipLaunchKernelGGL(xcd_map_kernel, dim3(64), dim3(64), 0, nullptr, d);
+        uint32_t h[64];
+        hipError_t e = hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost);
+        (void)hipFree(d);
+        if (e != hipSuccess) return MINT_ERR_HIP;
+        uint32_t mask = 0;
+        for (uint32_t v : h) mask |= 1u << (v & 31u);
+        *xcds = __builtin_popcount(mask);
+    }
+    return MINT_OK;
+}
+
+int mint_xcd_map(int blocks, void* out, void* stream) {
+    if (blocks <= 0 || !out) return MINT_ERR_ARG;
+    hipLaunchKernelGGL(xcd_map_kernel, dim3((unsigned)blocks), dim3(64), 0, as_stream(stream),
+                       static_cast<uint32_t*>(out));
+    return launch_status();
+}
+
+int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int threads,
+                     void* stream) {
+    if (nbytes == 0) return MINT_OK;
+    if (!src || !dst) return MINT_ERR_ARG;
+    if (!aligned16(src) || !aligned16(dst)) return MINT_ERR_ALIGN;
+    if (threads <= 0) threads = 512;
+    if (threads % 64 || threads > 1024) return MINT_ERR_ARG;
+    if (blocks <= 0) {
+        blocks = device_cus() * (2048 / threads);
+        if (blocks <= 0) return MINT_ERR_HIP;
+    }
+    const uint64_t need = (nbytes / 16 + (uint64_t)threads - 1) / (uint64_t)threads;
+    if ((uint64_t)blocks > need) blocks = need ? (int)need : 1;
+    hipLaunchKernelGGL(copy_simple_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0,
+                       as_stream(stream), static_cast<const uint8_t*>(src),
+                       static_cast<uint8_t*>(dst), (uint64_t)nbytes);
+    return launch_status();
+}
+
+size_t mint_ll128_packed_bytes(size_t nbytes, int layout) {
+    if (layout == MINT_LAYOUT_PAIR) return (nbytes + 119) / 120 * 128;
+    return (nbytes + 959) / 960 * 1024;
+}
+
+int mint_ll128_pack(const void* raw, void* msg, size_t nbytes, uint64_t flag_base,
+                    uint64_t flag_stride, int layout, void* stream) {
+    if (layout != MINT_LAYOUT_PAIR && layout != MINT_LAYOUT_WAVE64) return MINT_ERR_ARG;
+    if (nbytes == 0) return MINT_OK;
+    if (!raw || !msg) return MINT_ERR_ARG;
+    if (!aligned16(raw) || !aligned16(msg)) return MINT_ERR_ALIGN;
+    const uint64_t lines = mint_ll128_packed_bytes(nbytes, layout) / 128;
+    if (lines >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
+    const uint64_t waves = layout == MINT_LAYOUT_WAVE64 ? lines / 8 : (lines * 8 + 63) / 64;
+    uint64_t blocks = (waves + 3) / 4;
+    const uint64_t cap = (uint64_t)device_cus() * 8;
+    if (cap && blocks > cap) blocks = cap;
+    if (layout == MINT_LAYOUT_WAVE64)
+        hipLaunchKernelGGL(pack_wave64_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), static_cast<const uint8_t*>(raw),
+                           static_cast<uint8_t*>(msg), (uint64_t)nbytes, (uint32_t)(lines / 8),
+                           flag_base, flag_stride);
+    else
+        hipLaunchKernelGGL(pack_pair_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), static_cast<const uint8_t*>(raw),
+                           static_cast<uint8_t*>(msg), (uint64_t)nbytes, lines, flag_base,
+                           flag_stride);
+    return launch_status();
+}
+
+int mint_ll128_unpack(const void* msg, void* raw, size_t nbytes, uint64_t flag_base,
+                      uint64_t flag_stride, int layout, void* bad_flags, void* stream) {
+    if (layout != MINT_LAYOUT_PAIR && layout != MINT_LAYOUT_WAVE64) return MINT_ERR_ARG;
+    if (nbytes == 0) return MINT_OK;
+    if (!raw || !msg) return MINT_ERR_ARG;
+    if (!aligned16(raw) || !aligned16(msg)) return MINT_ERR_ALIGN;
+    const uint64_t lines = mint_ll128_packed_bytes(nbytes, layout) / 128;
+    if (lines >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
+    const uint64_t waves = layout == MINT_LAYOUT_WAVE64 ? lines / 8 : (lines * 8 + 63) / 64;
+    uint64_t blocks = (waves + 3) / 4;
+    const uint64_t cap = (uint64_t)device_cus() * 8;
+    if (cap && blocks > cap) blocks = cap;
+    if (layout == MINT_LAYOUT_WAVE64)
+        hipLaunchKernelGGL(unpack_wave64_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), static_cast<const uint8_t*>(msg),
+                           static_cast<uint8_t*>(raw), (uint64_t)nbytes, (uint32_t)(lines / 8),
+                           flag_base, flag_stride, static_cast<unsigned long long*>(bad_flags));
+    else
+        hipLaunchKernelGGL(unpack_pair_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                           as_stream(stream), static_cast<const uint8_t*>(msg),
+                           static_cast<uint8_t*>(raw), (uint64_t)nbytes, lines, flag_base,
+                           flag_stride, static_cast<unsigned long long*>(bad_flags));
+    return launch_status();
+}
+
+int mint_elementwise_sum(const void* a, const void* b, void* out, size_t nelem, int dtype,
+                         void* stream) {
+    if (dtype < MINT_F16 || dtype > MINT_F32) return MINT_ERR_ARG;
+    if (nelem == 0) return MINT_OK;
+    if (!a || !b || !out) return MINT_ERR_ARG;
+    if (!aligned16(a) || !aligned16(b) || !aligned16(out)) return MINT_ERR_ALIGN;
+    const uint64_t nbytes = (uint64_t)nelem * (dtype == MINT_F32 ? 4u : 2u);
+    uint64_t blocks = (nbytes / 16 + 255) / 256;
+    const uint64_t cap = (uint64_t)device_cus() * 8;
+    if (blocks == 0) blocks = 1;
+    if (cap && blocks > cap) blocks = cap;
+    const uint8_t* pa = static_cast<const uint8_t*>(a);
+    const uint8_t* pb = static_cast<const uint8_t*>(b);
+    uint8_t* po = static_cast<uint8_t*>(out);
+    switch (dtype) {
+        case MINT_F16:
+            hipLaunchKernelGGL(sum_kernel<DT_F16>, dim3((unsigned)blocks), dim3(256), 0,
+                               as_stream(stream), pa, pb, po, nbytes);
+            break;
+        case MINT_BF16:
+            hipLaunchKernelGGL(sum_kernel<DT_BF16>, dim3((unsigned)blocks), dim3(256), 0,
+                               as_stream(stream), pa, pb, po, nbytes);
+            break;
+        default:
+            hipLaunchKernelGGL(sum_kernel<DT_F32>, dim3((unsigned)blocks), dim3(256), 0,
+                               as_stream(stream), pa, pb, po, nbytes);
+    }
+    return launch_status();
+}
+
+size_t mint_ring_staging_bytes(const mint_ring_op* op) {
+    Plan plan;
+    if (make_plan(op, &plan) != MINT_OK) return 0;
+    return (size_t)plan.args.credit_off +
+           (size_t)plan.args.pipes * (size_t)plan.args.waves * kCreditStride;
+}
+
+int mint_ring_grid_blocks(const mint_ring_op* op) {
+    Plan plan;
+    const int err = make_plan(op, &plan);
+    return err != MINT_OK ? err : plan.blocks;
+}
+
+int mint_ring_launch(const mint_ring_op* op, void* stream) {
+    Plan plan;
+    const int err = make_plan(op, &plan);
+    if (err != MINT_OK) return err;
+    if (plan.empty) return MINT_OK;
+    return op->protocol == MINT_PROTO_LL128
+               ? launch_ring_dt<PROTO_LL128>(plan, op->dtype, op->cache_policy, as_stream(stream))
+               : launch_ring_dt<PROTO_SIMPLE>(plan, op->dtype, op->cache_policy, as_stream(stream));
+}
+
+int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,
+                         int cache_policy, int placement, uint32_t flag_epoch,
+                         uint32_t spin_budget, void* counters, void* stream) {
+    if (!staging || !counters || pairs <= 0 || iters <= 0 || flag_epoch == 0) return MINT_ERR_ARG;
+    if (!aligned16(staging)) return MINT_ERR_ALIGN;
+    if (cache_policy != 0 && cache_policy != 1) return MINT_ERR_ARG;
+    const size_t need = (size_t)pairs * (kProbeDepth * kBlockMsg + 128u);
+    if (staging_bytes < need || need >= (1ull << 31)) return MINT_ERR_ARG;
+    const int wpb = 4, pair_blocks = (pairs + wpb - 1) / wpb, blocks = 2 * pair_blocks;
+    auto kernel = cache_policy == 0 ? torn_probe_kernel<CP_AGENT> : torn_probe_kernel<CP_SYSTEM>;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess)
+        return MINT_ERR_HIP;
+    if (blocks > per_cu * device_cus()) return MINT_ERR_RESIDENCY;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<uint8_t*>(staging), (uint32_t)pairs, (uint32_t)iters, placement,
+                       flag_epoch, spin_budget ? spin_budget : kDefaultSpinBudget,
+                       static_cast<unsigned long long*>(counters));
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,56 @@
+"""Host handles on the device primitives.
+
+The reference's ``primitive.py`` holds PTX device functions; their CDNA4
+counterparts are in ``csrc/primitive.hpp``.  What can be called from the host
+is exposed here so each primitive can be tested by itself: the 128-bit
+load/store pair as a copy (``load128``/``store128``, ``primitive.py:180-203``)
+and the reduce operator (``SumFP16``, ``primitive.py:232-247``) for f16, bf16
+and f32.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .common import DTYPE_CODE
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def copy128(src: torch.Tensor, dst: torch.Tensor, blocks: int = 0, threads: int = 0) -> None:
+    """dst <- src with 16-byte loads / stores per lane."""
+    n = src.numel() * src.element_size()
+    if n != dst.numel() * dst.element_size():
+        raise ValueError("size mismatch")
+    with torch.cuda.device(src.device):
+        _lib.check(_lib.lib().mint_copy_simple(src.data_ptr(), dst.data_ptr(), n, blocks, threads,
+                                               _stream(src)), "mint_copy_simple")
+
+
+def Sum(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Elementwise ``rn(a + b)``, one rounding, by the ring kernels' own adder."""
+    if a.dtype not in DTYPE_CODE or a.dtype != b.dtype or a.numel() != b.numel():
+        raise ValueError("Sum needs two f16 / bf16 / f32 tensors of one shape")
+    if out is None:
+        out = torch.empty_like(a)
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.lib().mint_elementwise_sum(a.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                                   a.numel(), DTYPE_CODE[a.dtype], _stream(a)),
+                   "mint_elementwise_sum")
+    return out
+
+
+def SumFP16(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    if a.dtype != torch.float16:
+        raise ValueError("SumFP16 takes float16 tensors")
+    return Sum(a, b)
+
+
+def xcd_map(blocks: int, device="cuda:0") -> torch.Tensor:
+    """XCD each of ``blocks`` consecutive thread blocks lands on."""
+    out = torch.empty(blocks, dtype=torch.int32, device=device)
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.lib().mint_xcd_map(blocks, out.data_ptr(), _stream(out)), "mint_xcd_map")
+    return out

@@ -1,0 +1,150 @@
+/* Integer-only C restatement of the LL128 codec, of the element addition and
+ * of the ring reduce-scatter walked hop by hop through the wire format.
+ *
+ * TEST INFRASTRUCTURE ONLY: built into oracle/liboracle_c.so by oracle/Makefile
+ * and loaded by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg
+ * of bench.py.  The shipped library never links or loads it.
+ *
+ * It is written line by line (no index tables) so that it is an independent
+ * derivation from oracle/ll128.py, which is table driven.
+ *
+ * Reference semantics restated:
+ *   line format      protocol.py:42-48   (128 B = 120 B payload + 8 B flag)
+ *   pair layout      protocol.py:57-100,132-137 (load/save/send_ll128)
+ *   line numbers     2_sendrecv_indirect.py:61,76-77,93
+ *   fp16 addition    primitive.py:232-247 (add.f16x2: RNE, subnormals kept)
+ *   reduce order     7_reducescatter.py:54-73, protocol.py:150-155
+ * The wave64 layout is the 64-lane redesign described in oracle/ll128.py.
+ */
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+enum { LAYOUT_PAIR = 0, LAYOUT_WAVE64 = 1 };
+enum { DT_F16 = 0, DT_BF16 = 1, DT_F32 = 2 };
+
+static size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+
+size_t ref_line_count(size_t n, int layout) {
+    return layout == LAYOUT_PAIR ? ceil_div(n, 120) : ceil_div(n, 960) * 8;
+}
+
+/* copy raw[off, off+len) into dst, zero beyond n */
+static void take(const uint8_t *raw, size_t n, size_t off, size_t len, uint8_t *dst) {
+    size_t have = off < n ? (n - off < len ? n - off : len) : 0;
+    if (have) memcpy(dst, raw + off, have);
+    if (have < len) memset(dst + have, 0, len - have);
+}
+
+/* write src[0,len) to raw[off, off+len), dropping what lies beyond n */
+static void give(uint8_t *raw, size_t n, size_t off, size_t len, const uint8_t *src) {
+    size_t have = off < n ? (n - off < len ? n - off : len) : 0;
+    if (have) memcpy(raw + off, src, have);
+}
+
+static void put_flag(uint8_t *line, uint64_t f) {
+    for (int i = 0; i < 8; ++i) line[120 + i] = (uint8_t)(f >> (8 * i));
+}
+static uint64_t get_flag(const uint8_t *line) {
+    uint64_t f = 0;
+    for (int i = 0; i < 8; ++i) f |= (uint64_t)line[120 + i] << (8 * i);
+    return f;
+}
+
+void ref_pack(const uint8_t *raw, size_t n, uint64_t flag_base, uint64_t flag_stride,
+              int layout, uint8_t *msg) {
+    size_t lines = ref_line_count(n, layout);
+    for (size_t L = 0; L < lines; ++L) {
+        uint8_t *line = msg + L * 128;
+        if (layout == LAYOUT_PAIR) {
+            size_t base = (L / 2) * 240;
+            if (L % 2 == 0) {
+                take(raw, n, base, 120, line);
+            } else {
+                take(raw, n, base + 128, 112, line);
+                take(raw, n, base + 120, 8, line + 112);
+            }
+        } else {
+            size_t base = (L / 8) * 960, j = L % 8;
+            take(raw, n, base + 112 * j, 112, line);
+            take(raw, n, base + 896 + 8 * j, 8, line + 112);
+        }
+        put_flag(line, flag_base + L * flag_stride);
+    }
+}
+
+size_t ref_unpack(const uint8_t *msg, size_t n, uint64_t flag_base, uint64_t flag_stride,
+                  int layout, uint8_t *raw) {
+    size_t lines = ref_line_count(n, layout), bad = 0;
+    for (size_t L = 0; L < lines; ++L) {
+        const uint8_t *line = msg + L * 128;
+        if (get_flag(line) != flag_base + L * flag_stride) ++bad;
+        if (layout == LAYOUT_PAIR) {
+            size_t base = (L / 2) * 240;
+            if (L % 2 == 0) {
+                give(raw, n, base, 120, line);
+            } else {
+                give(raw, n, base + 128, 112, line);
+                give(raw, n, base + 120, 8, line + 112);
+            }
+        } else {
+            size_t base = (L / 8) * 960, j = L % 8;
+            give(raw, n, base + 112 * j, 112, line);
+            give(raw, n, base + 896 + 8 * j, 8, line + 112);
+        }
+    }
+    return bad;
+}
+
+/* Soft-float addition, round to nearest even, for a binary format with E
+ * exponent bits and M fraction bits (binary16: 5/10, bfloat16: 8/7).
+ * NaN results are the canonical quiet NaN (sign 0). */
+static uint32_t sf_add(uint32_t a, uint32_t b, int E, int M) {
+    const uint32_t emax = (1u << E) - 1, fmask = (1u << M) - 1;
+    uint32_t sa = a >> (E + M), ea = (a >> M) & emax, fa = a & fmask;
+    uint32_t sb = b >> (E + M), eb = (b >> M) & emax, fb = b & fmask;
+    const uint32_t qnan = (emax << M) | (1u << (M - 1));
+    if ((ea == emax && fa) || (eb == emax && fb)) return qnan;
+    if (ea == emax) return (eb == emax && sa != sb) ? qnan : a;
+    if (eb == emax) return b;
+    int xa = ea ? (int)ea : 1, xb = eb ? (int)eb : 1;
+    uint64_t va = (uint64_t)(ea ? fa | (1u << M) : fa) << 3;
+    uint64_t vb = (uint64_t)(eb ? fb | (1u << M) : fb) << 3;
+    if (xa < xb || (xa == xb && va < vb)) {
+        int tx = xa; xa = xb; xb = tx;
+        uint64_t tv = va; va = vb; vb = tv;
+        uint32_t ts = sa; sa = sb; sb = ts;
+    }
+    int d = xa - xb;
+    if (d > 0) {
+        if (d >= 40) vb = vb != 0;
+        else vb = (vb >> d) | ((vb & ((1ull << d) - 1)) != 0);
+    }
+    uint64_t v = sa == sb ? va + vb : va - vb;
+    int x = xa;
+    if (v == 0) return sa == sb ? sa << (E + M) : 0;
+    if (v >> (M + 4)) { v = (v >> 1) | (v & 1); ++x; }
+    while (x > 1 && !(v >> (M + 3))) { v <<= 1; --x; }
+    uint32_t g = (uint32_t)(v & 7), lsb = (uint32_t)(v >> 3) & 1;
+    v >>= 3;
+    if (g > 4 || (g == 4 && lsb)) ++v;
+    if (v >> (M + 1)) { v >>= 1; ++x; }
+    uint32_t e = (v >> M) ? (uint32_t)x : 0;
+    if (e >= emax) return (sa << (E + M)) | (emax << M);
+    return (sa << (E + M)) | (e << M) | ((uint32_t)v & fmask);
+}
+
+uint16_t ref_add_f16(uint16_t a, uint16_t b) { return (uint16_t)sf_add(a, b, 5, 10); }
+uint16_t ref_add_bf16(uint16_t a, uint16_t b) { return (uint16_t)sf_add(a, b, 8, 7); }
+
+/* out = rn(a + b) elementwise; nelem elements of the given dtype */
+void ref_add(const void *a, const void *b, void *out, size_t nelem, int dtype) {
+    if (dtype == DT_F32) {
+        const float *x = a, *y = b; float *o = out;
+        for (size_t i = 0; i < nelem; ++i) o[i] = x[i] + y[i];
+    } else {
+        const uint16_t *x = a, *y = b; uint16_t *o = out;
+        int E = dtype == DT_F16 ? 5 : 8, M = dtype == DT_F16 ? 10 : 7;
+        for (size_t i = 0; i < nelem; ++i) o[i] = (uint16_t)sf_add(x[i], y[i], E, M);
+    }
+}
