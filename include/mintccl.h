@@ -28,6 +28,7 @@ extern "C" {
 #define MINT_MAX_RANKS 8
 #define MINT_LINE_BYTES 128u     /* protocol.py:47 BYTES_LL128_MSG */
 #define MINT_LINE_PAYLOAD 120u   /* protocol.py:48 BYTES_LL128_RAW */
+#define MINT_SECTOR_BYTES 64u    /* unit that becomes visible as a whole */
 #define MINT_BLOCK_LINES 8u      /* lines one 64-lane access carries */
 #define MINT_BLOCK_MSG 1024u
 #define MINT_BLOCK_RAW 960u
@@ -83,14 +84,16 @@ typedef struct {
     uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE: bytes of the buffer;
                               ALLGATHER/REDUCESCATTER: bytes of one row */
     uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER: bytes between rows */
-    uint32_t slot_bytes;   /* staging bytes of one step over all channels */
+    uint32_t slot_bytes;   /* staging bytes of one step over all pipelines;
+                              multiple of 1024, >= 1024 per pipeline */
     uint32_t nslots;       /* slots in the circular staging buffer */
     uint32_t waves_per_channel_group; /* wave-channels per (pipeline, hop) */
     uint32_t threads_per_block;       /* multiple of 64 */
     int32_t placement;     /* mint_placement */
     int32_t cache_policy;  /* 0 agent scope (sc1), 1 system scope (sc0 sc1) */
-    uint32_t flag_epoch;   /* must differ from every earlier launch that used
-                              the same staging memory; never 0 */
+    uint32_t flag_epoch;   /* 1..4095; must differ from every earlier launch
+                              that used the same staging memory since that
+                              memory was last zeroed */
     uint32_t spin_budget;  /* polls before a wait gives up; 0 = default */
     uint64_t status;       /* device address of MINT_STATUS_WORDS uint64 */
     uint32_t debug_skip_origin; /* testing: origin hop sends nothing */
@@ -115,7 +118,11 @@ int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int 
                      void* stream);
 
 /* Standalone LL128 codec (load_ll128 + send_ll128 / recv_ll128 + save_ll128,
- * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride.
+ * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride:
+ * MINT_LAYOUT_PAIR is the reference's wire format (120 payload bytes, then the
+ * flag as 8 little-endian bytes); MINT_LAYOUT_WAVE64 is the format the ring
+ * kernels use (per 64-byte sector 60 payload bytes, then the low 32 bits of
+ * the flag).
  * msg must hold mint_ll128_packed_bytes(nbytes, layout).  bad_flags (device
  * uint64, may be 0) is incremented once per line whose flag is not the
  * expected one. */
@@ -137,13 +144,18 @@ int mint_ring_grid_blocks(const mint_ring_op* op);
 /* Validate and enqueue one fused launch that runs every rank's kernel. */
 int mint_ring_launch(const mint_ring_op* op, void* stream);
 
-/* Torn-line probe: `pairs` producer wavefronts each rewrite one 1 KiB block
- * `iters` times with lines whose payload is a function of the flag; the
- * paired consumer wavefronts poll until the flag appears and count lines
- * whose payload does not belong to the flag.  counters: device uint64[4] =
- * {lines checked, torn lines, polls, timeouts}. */
+/* Torn-line probe: `pairs` producer wavefronts each rewrite 1 KiB blocks of
+ * their own `iters` times; every 64-byte sector carries a tag and a payload
+ * that is a function of the tag.  The paired consumer wavefronts poll until
+ * the tags appear and count 128-byte lines holding bytes that do not belong to
+ * the tag.  per_sector = 1: all 16 sector tags of a block are tested (the ring
+ * kernels' format); per_sector = 0: only the tag of the second sector of each
+ * line is tested (one flag per 128-byte line, the reference's assumption,
+ * protocol.py:31-35).  counters: device uint64[8] = {lines checked, torn
+ * lines, polls, timeouts, torn lines whose first sector alone was stale, 0..}.
+ * flag_epoch is 1..4095. */
 int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,
-                         int cache_policy, int placement, uint32_t flag_epoch,
+                         int cache_policy, int placement, int per_sector, uint32_t flag_epoch,
                          uint32_t spin_budget, void* counters, void* stream);
 
 #ifdef __cplusplus

@@ -17,6 +17,7 @@ SRC = os.path.join(_PKG, "csrc", "mintccl.hip")
 
 MAX_RANKS = 8
 STATUS_WORDS = 4
+MAX_EPOCH = 4095          # sector tags carry a 12-bit launch epoch
 
 OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6
 LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
@@ -72,7 +73,7 @@ SYMBOLS = {
     "mint_ring_staging_bytes": (_sz, [_opp]),
     "mint_ring_grid_blocks": (_i, [_opp]),
     "mint_ring_launch": (_i, [_opp, _vp]),
-    "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
+    "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }
 
 _lib = None

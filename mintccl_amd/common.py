@@ -226,9 +226,9 @@ class VirtualComm:
         d.count_bytes, d.row_stride = count_bytes, row_stride
         d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
         pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER) else 1
-        if self.slot_bytes % (pipes * 1024):
-            raise ValueError("slot size must be a multiple of pipelines x 1 KiB")
-        step_blocks = self.slot_bytes // pipes // 1024
+        step_blocks = self.slot_bytes // 1024 // pipes
+        if self.slot_bytes % 1024 or step_blocks == 0:
+            raise ValueError("slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
         d.waves_per_channel_group = _largest_divisor_at_most(
             step_blocks, max(1, self.waves_per_rank // pipes))
         d.threads_per_block = self.threads_per_block
@@ -240,6 +240,11 @@ class VirtualComm:
 
     def launch(self, d: _lib.RingOp) -> None:
         """Enqueue on the current stream; never synchronises."""
+        # sector tags hold 12 bits of epoch: when the counter wraps, staging is
+        # cleared (a stream-ordered fill) so that no tag of an old launch survives
+        if self.epoch >= _lib.MAX_EPOCH:
+            self.staging.zero_()
+            self.epoch = 0
         self.epoch += 1
         d.flag_epoch = self.epoch
         self.last_grid = self._lib.mint_ring_grid_blocks(d)

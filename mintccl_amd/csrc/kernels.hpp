@@ -38,8 +38,9 @@ __global__ void __launch_bounds__(256) pack_wave64_kernel(const uint8_t* __restr
     const uint32_t wave = blockIdx.x * (blockDim.x >> 6) + (uint32_t)wave_in_block();
     for (uint32_t g = wave; g < nblocks; g += waves) {
         u32x4 v = ll_load_raw(raw, nbytes, g, m);
-        const uint64_t flag = flag_base + ((uint64_t)g * 8u + m.line) * flag_stride;
-        if (m.flag_lane) { v.z = (uint32_t)flag; v.w = (uint32_t)(flag >> 32); }
+        // line = two sectors; both carry the low 32 bits of the line's flag
+        const uint64_t flag = flag_base + ((uint64_t)g * 8u + (m.sector >> 1)) * flag_stride;
+        if (m.flag_lane) v.w = (uint32_t)flag;
         *reinterpret_cast<u32x4*>(msg + (uint64_t)g * kBlockMsg + m.lane * 16u) = v;
     }
 }
@@ -55,11 +56,14 @@ __global__ void __launch_bounds__(256) unpack_wave64_kernel(const uint8_t* __res
     uint32_t bad = 0;
     for (uint32_t g = wave; g < nblocks; g += waves) {
         u32x4 v = *reinterpret_cast<const u32x4*>(msg + (uint64_t)g * kBlockMsg + m.lane * 16u);
-        const uint64_t flag = flag_base + ((uint64_t)g * 8u + m.line) * flag_stride;
-        if (m.flag_lane && (v.z != (uint32_t)flag || v.w != (uint32_t)(flag >> 32))) ++bad;
+        const uint64_t flag = flag_base + ((uint64_t)g * 8u + (m.sector >> 1)) * flag_stride;
+        // a line is bad if either of its two sector tags is: pair up the
+        // flag lanes of a line through the ballot, count once per line
+        const uint64_t wrong = __ballot(m.flag_lane && v.w != (uint32_t)flag);
+        for (uint32_t j = 0; j < 8u; ++j) bad += ((wrong >> (8u * j)) & 0xFFull) ? 1u : 0u;
         ll_save_raw(raw, nbytes, g, m, v);
     }
-    if (bad && bad_flags) atomicAdd(bad_flags, (unsigned long long)bad);
+    if (bad && bad_flags && lane_id() == 0) atomicAdd(bad_flags, (unsigned long long)bad);
 }
 
 // ---- LL128 codec, reference pair layout: one thread per 16-byte message
@@ -136,17 +140,21 @@ __global__ void xcd_map_kernel(uint32_t* out) {
 }
 
 // ---- torn-line probe --------------------------------------------------------
-// The payload of a line is a function of its flag, so a consumer that sees
-// the flag can tell whether the other 120 bytes belong to it.
-__device__ __forceinline__ uint32_t probe_word(uint32_t flag_lo, uint32_t lane, uint32_t d) {
-    return (flag_lo * 2654435761u) ^ (lane * 0x9E3779B1u + d * 0x85EBCA77u + 0x1234567u);
+// The payload of a sector is a function of its tag, so a consumer that sees
+// the tag can tell whether the other bytes belong to it.  `per_sector` = 1 is
+// the format the ring kernels use (a tag in every 64-byte sector, all 16
+// tested); `per_sector` = 0 tests only the tag of the second sector of each
+// 128-byte line, which is what a one-flag-per-line format amounts to.
+__device__ __forceinline__ uint32_t probe_word(uint32_t tag, uint32_t lane, uint32_t d) {
+    return (tag * 2654435761u) ^ (lane * 0x9E3779B1u + d * 0x85EBCA77u + 0x1234567u);
 }
 constexpr uint32_t kProbeDepth = 4;   // blocks per pair, reused round-robin
 
 template <int CP>
 __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint32_t pairs,
                                                          uint32_t iters, int placement,
-                                                         uint32_t epoch, uint32_t budget,
+                                                         int per_sector, uint32_t epoch,
+                                                         uint32_t budget,
                                                          unsigned long long* counters) {
     const LaneMap m;
     const uint32_t wpb = blockDim.x >> 6;
@@ -160,12 +168,10 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
     const Window win(staging, data_bytes);
     uint64_t* tail = reinterpret_cast<uint64_t*>(staging + data_bytes + (uint64_t)pair * 128u);
     const uint64_t flag_hi = (uint64_t)epoch << 32;
-    unsigned long long checked = 0, torn = 0, polls = 0, timeouts = 0;
-    uint32_t seen = 0;
+    unsigned long long checked = 0, torn = 0, polls = 0, timeouts = 0, first_half = 0;
     for (uint32_t t = 0; t < iters; ++t) {
         const uint32_t off = (pair * kProbeDepth + t % kProbeDepth) * kBlockMsg;
-        const uint64_t flag = flag_hi | ((uint64_t)t * 8u + m.line + 1u);
-        const uint32_t flo = (uint32_t)flag;
+        const uint32_t tag = (epoch << 20) | ((t + 1u) & 0xFFFFFu);
         if (producer) {
             if (t >= kProbeDepth) {
                 bool ok = false;
@@ -173,38 +179,44 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
                     uint64_t v = ld64_agent(tail);
                     uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
                     uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-                    if (hi == epoch && lo >= t - kProbeDepth + 1) { ok = true; seen = lo; break; }
+                    if (hi == epoch && lo >= t - kProbeDepth + 1) { ok = true; break; }
                     __builtin_amdgcn_s_sleep(1);
                 }
                 if (!ok) { ++timeouts; break; }
             }
-            u32x4 v = {probe_word(flo, m.lane, 0), probe_word(flo, m.lane, 1),
-                       probe_word(flo, m.lane, 2), probe_word(flo, m.lane, 3)};
-            ll_send<CP>(win, off, v, flag, m);
+            u32x4 v = {probe_word(tag, m.lane, 0), probe_word(tag, m.lane, 1),
+                       probe_word(tag, m.lane, 2), probe_word(tag, m.lane, 3)};
+            ll_send<CP>(win, off, v, tag, m);
         } else {
             u32x4 v; bool ok = false;
             for (uint32_t spins = 0; spins <= budget; ++spins) {
                 compiler_fence();
                 ++polls;
-                if (ll_poll<CP>(win, off, flag, m, v)) { ok = true; break; }
+                v = ld128<CP>(win, off + m.lane * 16u);
+                const bool tested = m.flag_lane && (per_sector || (m.sector & 1u));
+                if (wave_all(!tested || v.w == tag)) { ok = true; break; }
                 __builtin_amdgcn_s_sleep(1);
             }
             if (!ok) { ++timeouts; break; }
-            bool bad = v.x != probe_word(flo, m.lane, 0) || v.y != probe_word(flo, m.lane, 1);
-            if (!m.flag_lane)
-                bad = bad || v.z != probe_word(flo, m.lane, 2) || v.w != probe_word(flo, m.lane, 3);
+            bool bad = v.x != probe_word(tag, m.lane, 0) || v.y != probe_word(tag, m.lane, 1) ||
+                       v.z != probe_word(tag, m.lane, 2);
+            bad = bad || (m.flag_lane ? v.w != tag : v.w != probe_word(tag, m.lane, 3));
             const uint64_t mask = __ballot(bad);
-            for (uint32_t j = 0; j < 8u; ++j) torn += ((mask >> (8u * j)) & 0xFFull) ? 1u : 0u;
+            for (uint32_t j = 0; j < 8u; ++j) {
+                const uint32_t line = (uint32_t)(mask >> (8u * j)) & 0xFFu;
+                torn += line ? 1u : 0u;
+                first_half += line == 0x0Fu ? 1u : 0u;   // exactly the first sector stale
+            }
             checked += 8u;
             if (lane_id() == 0) st64_agent(tail, flag_hi | (uint64_t)(t + 1));
         }
     }
-    (void)seen;
     if (lane_id() == 0) {
         if (checked) atomicAdd(counters + 0, checked);
         if (torn) atomicAdd(counters + 1, torn);
         if (polls) atomicAdd(counters + 2, polls);
         if (timeouts) atomicAdd(counters + 3, timeouts);
+        if (first_half) atomicAdd(counters + 4, first_half);
     }
 }
 

@@ -12,6 +12,8 @@ namespace {
 
 constexpr int kVersion = 100;   // 0.1.0
 constexpr uint32_t kDefaultSpinBudget = 4000000u;
+constexpr uint32_t kMaxEpoch = 4095u;          // 12 bits of every sector tag
+constexpr uint32_t kMaxSteps = (1u << 20) - 1; // 20 bits of every sector tag
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
@@ -45,7 +47,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
     if (op->cache_policy != 0 && op->cache_policy != 1) return MINT_ERR_ARG;
     if (op->placement != MINT_PLACE_SPREAD && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
-    if (op->flag_epoch == 0 || !op->status) return MINT_ERR_ARG;
+    if (op->flag_epoch == 0 || op->flag_epoch > kMaxEpoch || !op->status) return MINT_ERR_ARG;
     if (op->threads_per_block == 0 || op->threads_per_block % 64 || op->threads_per_block > 512)
         return MINT_ERR_ARG;
     if (op->nslots == 0 || op->slot_bytes == 0) return MINT_ERR_GEOMETRY;
@@ -125,9 +127,12 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     // geometry
     a.slot_bytes = op->slot_bytes;
     a.nslots = op->nslots;
-    if (op->slot_bytes % ((uint32_t)a.pipes * kBlockMsg)) return MINT_ERR_GEOMETRY;
-    a.step_msg = op->slot_bytes / (uint32_t)a.pipes;
-    a.step_blocks = a.step_msg / kBlockMsg;
+    // a slot is shared evenly by the pipelines, in whole 1 KiB blocks; what
+    // does not divide is left unused
+    if (op->slot_bytes % kBlockMsg) return MINT_ERR_GEOMETRY;
+    a.step_blocks = op->slot_bytes / kBlockMsg / (uint32_t)a.pipes;
+    if (a.step_blocks == 0) return MINT_ERR_GEOMETRY;
+    a.step_msg = a.step_blocks * kBlockMsg;
     if (op->waves_per_channel_group == 0 || a.step_blocks % op->waves_per_channel_group)
         return MINT_ERR_GEOMETRY;
     a.waves = (int)op->waves_per_channel_group;
@@ -137,6 +142,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     if (nblocks >= (1ull << 28)) return MINT_ERR_TOO_LARGE;
     a.nblocks = (uint32_t)nblocks;
     a.steps = (a.nblocks + a.step_blocks - 1) / a.step_blocks;
+    if (a.steps > kMaxSteps) return MINT_ERR_TOO_LARGE;
     a.credit_off = a.nslots * a.slot_bytes;
     a.epoch = op->flag_epoch;
     a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
@@ -364,9 +370,11 @@ int mint_ring_launch(const mint_ring_op* op, void* stream) {
 }
 
 int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,
-                         int cache_policy, int placement, uint32_t flag_epoch,
+                         int cache_policy, int placement, int per_sector, uint32_t flag_epoch,
                          uint32_t spin_budget, void* counters, void* stream) {
-    if (!staging || !counters || pairs <= 0 || iters <= 0 || flag_epoch == 0) return MINT_ERR_ARG;
+    if (!staging || !counters || pairs <= 0 || iters <= 0 || iters > (int)kMaxSteps ||
+        flag_epoch == 0 || flag_epoch > kMaxEpoch)
+        return MINT_ERR_ARG;
     if (!aligned16(staging)) return MINT_ERR_ALIGN;
     if (cache_policy != 0 && cache_policy != 1) return MINT_ERR_ARG;
     const size_t need = (size_t)pairs * (kProbeDepth * kBlockMsg + 128u);
@@ -379,7 +387,7 @@ int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int ite
     if (blocks > per_cu * device_cus()) return MINT_ERR_RESIDENCY;
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                        static_cast<uint8_t*>(staging), (uint32_t)pairs, (uint32_t)iters, placement,
-                       flag_epoch, spin_budget ? spin_budget : kDefaultSpinBudget,
+                       per_sector ? 1 : 0, flag_epoch, spin_budget ? spin_budget : kDefaultSpinBudget,
                        static_cast<unsigned long long*>(counters));
     return launch_status();
 }

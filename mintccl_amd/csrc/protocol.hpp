@@ -3,42 +3,50 @@
 // Reference: protocol.py.  There an 8-lane "workgroup" moves two 128-byte
 // lines per step (protocol.py:42-52) and lane 7 of each group carries 8
 // payload bytes plus the 8-byte flag (load_ll128 :57-85, save_ll128 :87-100,
-// recv_ll128 :102-130, send_ll128 :132-137, comp_ll128 :142-156).
+// recv_ll128 :102-130, send_ll128 :132-137, comp_ll128 :142-156).  That format
+// rests on a 128-byte store becoming visible as a whole (protocol.py:31-35).
+// On MI355X it does not: a consumer workgroup can see the second 64-byte
+// sector of a line (the one with the flag) while the first still holds the
+// previous occupant of the slot.  64-byte sectors were never seen torn.
 //
-// Here the unit is a *block*: one wavefront moves 8 lines (1 KiB of message,
+// So the line keeps its 128 bytes, 120 of payload and 8 of flag, but the flag
+// is a 32-bit tag stored once per 64-byte sector:
+//     [0,60) payload | [60,64) tag | [64,124) payload | [124,128) tag
+// and the unit is a *block*: one wavefront moves 8 lines (1 KiB of message,
 // 960 payload bytes) with a single 16-byte access per lane.
-//   lane l, l % 8 != 7 : aligned raw vector number  l - l / 8   (0..55)
-//   lane l = 8 j + 7   : raw bytes [896 + 8 j, 904 + 8 j) and the flag of line j
-// so a block is 60 aligned 16-byte raw vectors, and both the raw side and the
-// message side are touched by contiguous, 16-byte-aligned accesses; the flag
-// test is one 64-bit ballot.  The flag lanes read their 8 bytes with the same
-// 16-byte load as everybody else (vector 56 + j / 2, half j % 2): the
-// reference's own trick (protocol.py:74-82) widened to 64 lanes.
+//   lane l, l % 4 != 3 : aligned raw vector number  l - l / 4   (0..47)
+//   lane l = 4 i + 3   : raw bytes [768 + 12 i, 780 + 12 i) and the tag of
+//                        sector i
+// Both sides are touched by contiguous accesses; the flag test is one 64-bit
+// ballot.  A flag lane reads its 12 bytes with the same 16-byte load
+// instruction as everybody else, starting 4 bytes early (the reference's own
+// trick, protocol.py:74-82, widened to 64 lanes).
 #pragma once
 #include "primitive.hpp"
 
 namespace mint {
 
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+typedef u32x3 u32x3_a4 __attribute__((aligned(4)));
+
 constexpr uint32_t kLineBytes = 128, kLinePayload = 120;
 constexpr uint32_t kBlockMsg = 1024, kBlockRawLL = 960, kBlockRawSimple = 1024;
+constexpr uint32_t kFlagLaneRaw = 768;    // first raw byte carried by a flag lane
 
 // Per-lane constants of the wave64 layout.
 struct LaneMap {
     uint32_t lane;
-    uint32_t line;       // line of the block this lane belongs to (0..7)
+    uint32_t sector;     // 64-byte sector of the block this lane belongs to (0..15)
     bool flag_lane;
     uint32_t raw_off;    // first raw byte this lane carries, inside the block
-    uint32_t raw_len;    // 16, or 8 on flag lanes
-    uint32_t ld_off;     // aligned 16-byte vector the lane loads
-    bool hi_half;        // flag lanes: which half of that vector is theirs
+    uint32_t raw_len;    // 16, or 12 on flag lanes
     __device__ __forceinline__ LaneMap() {
         lane = (uint32_t)lane_id();
-        line = lane >> 3;
-        flag_lane = (lane & 7u) == 7u;
-        raw_off = flag_lane ? 896u + 8u * line : (lane - line) * 16u;
-        raw_len = flag_lane ? 8u : 16u;
-        ld_off = flag_lane ? (56u + (line >> 1)) * 16u : raw_off;
-        hi_half = flag_lane && (line & 1u);
+        sector = lane >> 2;
+        flag_lane = (lane & 3u) == 3u;
+        raw_off = flag_lane ? kFlagLaneRaw + 12u * sector : (lane - sector) * 16u;
+        raw_len = flag_lane ? 12u : 16u;
     }
 };
 
@@ -51,8 +59,13 @@ __device__ __forceinline__ u32x4 load_guarded(const uint8_t* base, uint64_t off,
     uint64_t have = nbytes - off;
     if (have >= len) {
         if (len == 16u) return *reinterpret_cast<const u32x4*>(base + off);
-        u32x2 h = *reinterpret_cast<const u32x2*>(base + off);
-        v.x = h.x; v.y = h.y;
+        if (len == 12u) {
+            u32x3 h = *reinterpret_cast<const u32x3_a4*>(base + off);
+            v.x = h.x; v.y = h.y; v.z = h.z;
+        } else {                                   // 8
+            u32x2 h = *reinterpret_cast<const u32x2*>(base + off);
+            v.x = h.x; v.y = h.y;
+        }
         return v;
     }
     uint32_t w[4] = {0u, 0u, 0u, 0u};
@@ -67,8 +80,13 @@ __device__ __forceinline__ void store_guarded(uint8_t* base, uint64_t off, uint3
     uint64_t have = nbytes - off;
     if (have >= len) {
         if (len == 16u) { *reinterpret_cast<u32x4*>(base + off) = v; return; }
-        u32x2 h = {v.x, v.y};
-        *reinterpret_cast<u32x2*>(base + off) = h;
+        if (len == 12u) {
+            u32x3 h = {v.x, v.y, v.z};
+            *reinterpret_cast<u32x3_a4*>(base + off) = h;
+        } else {                                   // 8
+            u32x2 h = {v.x, v.y};
+            *reinterpret_cast<u32x2*>(base + off) = h;
+        }
         return;
     }
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -78,14 +96,17 @@ __device__ __forceinline__ void store_guarded(uint8_t* base, uint64_t off, uint3
 
 // ---- wave64 LL128 block: raw side ----------------------------------------
 // load_ll128 (protocol.py:57-85): raw block g of a row -> registers.  On
-// flag lanes .x/.y hold the 8 payload bytes; .z/.w are don't-care.
+// flag lanes .x/.y/.z hold the 12 payload bytes; .w is don't-care.
 __device__ __forceinline__ u32x4 ll_load_raw(const uint8_t* row, uint64_t row_bytes, uint32_t g,
                                              const LaneMap& m) {
     const uint64_t base = (uint64_t)g * kBlockRawLL;
     u32x4 v;
     if (base + kBlockRawLL <= row_bytes) {       // wave-uniform
-        v = ld128_stream(row + base + m.ld_off);
-        if (m.hi_half) { v.x = v.z; v.y = v.w; }
+        // flag lanes start 4 bytes early so that all 64 lanes issue one
+        // 16-byte load that stays inside the block
+        const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
+        v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(row + base + off));
+        if (m.flag_lane) { v.x = v.y; v.y = v.z; v.z = v.w; }
     } else {
         v = load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
     }
@@ -99,8 +120,8 @@ __device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, ui
         if (!m.flag_lane) {
             st128_stream(row + base + m.raw_off, v);
         } else {
-            u32x2 h = {v.x, v.y};
-            st64_stream(row + base + m.raw_off, h);
+            u32x3 h = {v.x, v.y, v.z};
+            __builtin_nontemporal_store(h, reinterpret_cast<u32x3_a4*>(row + base + m.raw_off));
         }
     } else {
         store_guarded(row, base + m.raw_off, m.raw_len, row_bytes, v);
@@ -108,31 +129,25 @@ __device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, ui
 }
 
 // ---- wave64 LL128 block: message side ------------------------------------
-// Flag of line j of a block whose first line carries `first`.
-__device__ __forceinline__ uint64_t ll_line_flag(uint64_t first, uint64_t stride,
-                                                 const LaneMap& m) {
-    return first + (uint64_t)m.line * stride;
-}
-// send_ll128 (protocol.py:132-137): one 1 KiB store, flags riding in the
-// last 8 bytes of every line.
+// send_ll128 (protocol.py:132-137): one 1 KiB store, a tag riding in the
+// last 4 bytes of every 64-byte sector.
 template <int CP>
-__device__ __forceinline__ void ll_send(const Window& dst, uint32_t off, u32x4 v, uint64_t flag,
+__device__ __forceinline__ void ll_send(const Window& dst, uint32_t off, u32x4 v, uint32_t tag,
                                         const LaneMap& m) {
-    if (m.flag_lane) { v.z = (uint32_t)flag; v.w = (uint32_t)(flag >> 32); }
+    if (m.flag_lane) v.w = tag;
     st128<CP>(dst, off + m.lane * 16u, v);
 }
 // One poll of recv_ll128 (protocol.py:102-130): load the block, report whether
-// all 8 flags are the expected ones (64-lane ballot in place of any_sync).
+// all 16 sector tags are the expected one (64-lane ballot in place of any_sync).
 template <int CP>
-__device__ __forceinline__ bool ll_poll(const Window& src, uint32_t off, uint64_t flag,
+__device__ __forceinline__ bool ll_poll(const Window& src, uint32_t off, uint32_t tag,
                                         const LaneMap& m, u32x4& v) {
     v = ld128<CP>(src, off + m.lane * 16u);
-    const bool ok = !m.flag_lane || (v.z == (uint32_t)flag && v.w == (uint32_t)(flag >> 32));
-    return wave_all(ok);
+    return wave_all(!m.flag_lane || v.w == tag);
 }
-// comp_ll128 (protocol.py:142-156): own + received; the flag words of the
-// flag lanes are not data - ll_send overwrites them - so all four words are
-// added on every lane and no lane diverges.
+// comp_ll128 (protocol.py:142-156): own + received; the tag word of a flag
+// lane is not data - ll_send overwrites it - so all four words are added on
+// every lane and no lane diverges.
 template <int DT>
 __device__ __forceinline__ u32x4 ll_comp(u32x4 own, u32x4 received) {
     return add_rn<DT>(own, received);

@@ -22,10 +22,11 @@
 // pipelines, split evenly: step s of pipeline p lives at
 //     (s % nslots) * slot_bytes + p * (slot_bytes / P)
 // and inside it block i = k * W + w is wave-channel w's k-th block of the step.
-// Flags are (epoch << 32 | 1-based line number inside the row), unique over a
-// launch, so a slot is never cleared (the reference's idea,
-// 2_sendrecv_indirect.py:59-61); the epoch makes them unique across launches
-// as well.  Flow control is a consumer-owned credit word per wave-channel
+// Every 64-byte sector of step s carries the 32-bit tag (epoch << 20 | s + 1):
+// successive occupants of a slot differ in the step, launches differ in the
+// epoch, so a slot is never cleared (the reference's idea of a unique,
+// never-zero flag, 2_sendrecv_indirect.py:59-61); the caller clears staging
+// when its 12-bit epoch counter wraps.  Flow control is a consumer-owned credit word per wave-channel
 // ((epoch << 32) | steps consumed) that the upstream producer polls before it
 // reuses a slot - separate from the data lines, unlike wait/post_ll128 which
 // overload the flag word of slot 0.
@@ -146,14 +147,14 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + chan_off);
     uint64_t* nxt_head = nxt_tail + 16;
 
-    const uint64_t flag_hi = (uint64_t)a.epoch << 32;
+    const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
     const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
-    const uint32_t raw_per_block = PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
     uint32_t credits_seen = 0, head_seen = 0;
 
     for (uint32_t s = 0; s < a.steps; ++s) {
         const uint32_t slot_off = (s % a.nslots) * a.slot_bytes + (uint32_t)p * a.step_msg;
         const uint32_t g0 = s * a.step_blocks;
+        const uint32_t tag = (a.epoch << 20) | (s + 1u);
         if (role.send && s >= a.nslots) {
             if (!wait_count(nxt_tail, a.epoch, s - a.nslots + 1, credits_seen, a.spin_budget,
                             a.status, false)) {
@@ -203,9 +204,7 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
                             if (!(pending & (1u << u))) continue;
-                            const uint64_t first = flag_hi | ((uint64_t)g[u] * 8u + 1u);
-                            if (ll_poll<CP>(own, slot_off + idx[u] * kBlockMsg,
-                                            ll_line_flag(first, 1, m), m, r[u]))
+                            if (ll_poll<CP>(own, slot_off + idx[u] * kBlockMsg, tag, m, r[u]))
                                 pending &= ~(1u << u);
                         }
                         if (!pending) break;
@@ -250,16 +249,13 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
                 for (int u = 0; u < U; ++u) {
                     if (!valid[u]) continue;
                     if (PROTO == PROTO_LL128) {
-                        const uint64_t first = flag_hi | ((uint64_t)g[u] * 8u + 1u);
-                        ll_send<CP>(nxt, slot_off + idx[u] * kBlockMsg, v[u],
-                                    ll_line_flag(first, 1, m), m);
+                        ll_send<CP>(nxt, slot_off + idx[u] * kBlockMsg, v[u], tag, m);
                     } else {
                         st128<CP>(nxt, slot_off + idx[u] * kBlockMsg + m.lane * 16u, v[u]);
                     }
                 }
             }
         }
-        (void)raw_per_block;
         // post_ll128 (protocol.py:183-189): this wave-channel has taken every
         // line of step s out of its slot (the loads have returned: their
         // values were tested / used above).

@@ -19,16 +19,22 @@ bytes.  From ``load_ll128`` (``protocol.py:57-85``) and ``send_ll128``
 ``save_ll128`` (``protocol.py:87-100``) is the inverse.  Line numbers start at
 1 and are unique over a transfer (``2_sendrecv_indirect.py:61,93``).
 
-``LAYOUT_WAVE64`` - the format the HIP kernels use for staging.  One 64-lane
-wavefront moves a *block* of 8 lines with one 16-byte access per lane:
-960 raw bytes <-> 1024 message bytes.  Lane ``l`` with ``l % 8 != 7`` carries
-the aligned raw vector number ``l - l // 8`` (0..55); the flag lane of line
-``j`` (``l = 8 j + 7``) carries raw bytes ``[896 + 8 j, 904 + 8 j)`` and the
-flag.  So, inside block ``b`` (first line number ``f = base + 8 b``)::
+``LAYOUT_WAVE64`` - the format the HIP kernels use for staging.  On MI355X a
+128-byte store does not become visible as a whole (64-byte sectors do), so the
+8 flag bytes of a line are spent as one 32-bit tag per 64-byte sector::
 
-    msg[128 j      : 128 j + 112] = raw[112 j : 112 j + 112]
-    msg[128 j + 112: 128 j + 120] = raw[896 + 8 j : 904 + 8 j]
-    msg[128 j + 120: 128 j + 128] = LE64(f + j)            j = 0..7
+    line = [0,60) payload | [60,64) tag | [64,124) payload | [124,128) tag
+
+where tag = low 32 bits of the line's flag, little endian.  One 64-lane
+wavefront moves a *block* of 8 lines (16 sectors) with one 16-byte access per
+lane: 960 raw bytes <-> 1024 message bytes.  Lane ``l`` with ``l % 4 != 3``
+carries the aligned raw vector number ``l - l // 4`` (0..47); the flag lane of
+sector ``i`` (``l = 4 i + 3``) carries raw bytes ``[768 + 12 i, 780 + 12 i)``
+and the tag.  So, inside block ``b`` (first line number ``f = base + 8 b``)::
+
+    msg[64 i      : 64 i + 48] = raw[48 i : 48 i + 48]
+    msg[64 i + 48 : 64 i + 60] = raw[768 + 12 i : 780 + 12 i]
+    msg[64 i + 60 : 64 i + 64] = LE32(f + i // 2)          i = 0..15
 
 A buffer whose size is not a multiple of the unit is zero padded: the pair
 layout packs ``ceil(n / 120)`` lines, the wave64 layout ``ceil(n / 960)``
@@ -39,8 +45,8 @@ Pinning.  The closed-form maps below are checked in ``tests/test_oracle_ll128``
 against (i) per-lane simulations written independently from the register
 moves in the cited lines, (ii) the hand-computed known answer for raw = 0..239,
 f = 7, (iii) the integer-only C restatement ``ll128_ref.c``, and (iv) the
-invariants ``unpack(pack(x)) == x``, flags at bytes 120..127 of every line,
-packed size.  The reference holds no golden vectors for this path.
+invariants ``unpack(pack(x)) == x``, flags where the layout puts them in every
+line, packed size.  The reference holds no golden vectors for this path.
 """
 from __future__ import annotations
 
@@ -55,6 +61,8 @@ LANES_PER_LINE = 8        # protocol.py:44  WORKGROUP_SIZE
 PAIR_RAW = 2 * LINE_PAYLOAD        # 240
 PAIR_MSG = 2 * LINE_BYTES          # 256
 BLOCK_LINES = 8                    # lines per 64-lane access
+SECTOR_BYTES = 64                  # what becomes visible as a whole on MI355X
+BLOCK_SECTORS = 16
 BLOCK_RAW = BLOCK_LINES * LINE_PAYLOAD   # 960
 BLOCK_MSG = BLOCK_LINES * LINE_BYTES     # 1024
 
@@ -76,11 +84,12 @@ def pair_byte_map() -> np.ndarray:
 
 
 def wave64_byte_map() -> np.ndarray:
+    """message byte -> raw byte, or -(1 + line) for a byte of that line's tag."""
     m = np.empty(BLOCK_MSG, dtype=np.int64)
-    for j in range(BLOCK_LINES):
-        m[128 * j:128 * j + 112] = np.arange(112 * j, 112 * j + 112)
-        m[128 * j + 112:128 * j + 120] = np.arange(896 + 8 * j, 904 + 8 * j)
-        m[128 * j + 120:128 * j + 128] = -(1 + j)
+    for i in range(BLOCK_SECTORS):
+        m[64 * i:64 * i + 48] = np.arange(48 * i, 48 * i + 48)
+        m[64 * i + 48:64 * i + 60] = np.arange(768 + 12 * i, 780 + 12 * i)
+        m[64 * i + 60:64 * i + 64] = -(1 + i // 2)
     return m
 
 
@@ -110,6 +119,25 @@ def _flags(nlines: int, flag_base: int, flag_stride: int) -> np.ndarray:
             + np.arange(nlines, dtype=np.uint64) * np.uint64(flag_stride))
 
 
+def _put_flags(lines: np.ndarray, flags: np.ndarray, layout: int) -> None:
+    if layout == LAYOUT_PAIR:
+        lines[:, 120:128] = flags.astype("<u8").view(np.uint8).reshape(-1, 8)
+    else:
+        tag = (flags & np.uint64(0xFFFFFFFF)).astype("<u4").view(np.uint8).reshape(-1, 4)
+        lines[:, 60:64] = tag
+        lines[:, 124:128] = tag
+
+
+def _count_bad_flags(lines: np.ndarray, flags: np.ndarray, layout: int) -> int:
+    if layout == LAYOUT_PAIR:
+        got = lines[:, 120:128].copy().view("<u8").reshape(-1)
+        return int(np.count_nonzero(got != flags))
+    want = (flags & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+    a = lines[:, 60:64].copy().view("<u4").reshape(-1)
+    b = lines[:, 124:128].copy().view("<u4").reshape(-1)
+    return int(np.count_nonzero((a != want) | (b != want)))
+
+
 def pack(raw, flag_base: int = 1, layout: int = LAYOUT_PAIR,
          flag_stride: int = 1) -> np.ndarray:
     """raw bytes -> LL128 message bytes.
@@ -133,7 +161,7 @@ def pack(raw, flag_base: int = 1, layout: int = LAYOUT_PAIR,
     flags = np.zeros(nunits * ulines, dtype=np.uint64)
     flags[:nlines] = _flags(nlines, flag_base, flag_stride)
     lines = msg.reshape(nunits * ulines, LINE_BYTES)
-    lines[:, LINE_PAYLOAD:] = flags.astype("<u8").view(np.uint8).reshape(-1, 8)
+    _put_flags(lines, flags, layout)
     return lines[:nlines].reshape(-1).copy()
 
 
@@ -150,8 +178,7 @@ def unpack(msg, nbytes: int, flag_base: int = 1, layout: int = LAYOUT_PAIR,
     full = np.zeros(nunits * umsg, dtype=np.uint8)
     full[:nlines * LINE_BYTES] = msg[:nlines * LINE_BYTES]
     lines = full.reshape(nunits * ulines, LINE_BYTES)
-    got = lines[:nlines, LINE_PAYLOAD:].copy().view("<u8").reshape(-1)
-    bad = int(np.count_nonzero(got != _flags(nlines, flag_base, flag_stride)))
+    bad = _count_bad_flags(lines[:nlines], _flags(nlines, flag_base, flag_stride), layout)
     units = full.reshape(nunits, umsg)
     raw = np.zeros((nunits, uraw), dtype=np.uint8)
     data = bmap >= 0
@@ -214,17 +241,19 @@ def pair_lane_sim_unpack(msg256: np.ndarray) -> np.ndarray:
 def wave64_lane_sim_pack(raw960: np.ndarray, first_flag: int,
                          flag_stride: int = 1) -> np.ndarray:
     """One block, lane by lane, the way a 64-lane wavefront does it: data
-    lanes load the aligned 16-byte vector ``lane - lane // 8``; the flag lane
-    of line ``j`` loads vector ``56 + j // 2`` and keeps its half ``j % 2``."""
+    lanes load the aligned 16-byte vector ``lane - lane // 4``; the flag lane
+    of sector ``i`` loads 16 bytes starting 4 bytes before its 12 and shifts."""
     msg = np.zeros(1024, dtype=np.uint8)
     for lane in range(64):
-        j, k = divmod(lane, 8)
-        if k != 7:
-            vec = lane - j
+        i, q = divmod(lane, 4)
+        if q != 3:
+            vec = lane - i
             msg[lane * 16:lane * 16 + 16] = raw960[vec * 16:vec * 16 + 16]
         else:
-            vec = 56 + j // 2
-            half = raw960[vec * 16 + 8 * (j % 2):vec * 16 + 8 * (j % 2) + 8]
-            msg[lane * 16:lane * 16 + 8] = half
-            msg[lane * 16 + 8:lane * 16 + 16] = _b64(first_flag + j * flag_stride)
+            start = 768 + 12 * i - 4
+            loaded = raw960[start:start + 16]
+            msg[lane * 16:lane * 16 + 12] = loaded[4:16]
+            tag = (first_flag + (i // 2) * flag_stride) & 0xFFFFFFFF
+            msg[lane * 16 + 12:lane * 16 + 16] = np.frombuffer(
+                int(tag).to_bytes(4, "little"), dtype=np.uint8)
     return msg

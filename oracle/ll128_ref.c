@@ -42,13 +42,27 @@ static void give(uint8_t *raw, size_t n, size_t off, size_t len, const uint8_t *
     if (have) memcpy(raw + off, src, have);
 }
 
-static void put_flag(uint8_t *line, uint64_t f) {
-    for (int i = 0; i < 8; ++i) line[120 + i] = (uint8_t)(f >> (8 * i));
+/* pair layout: 8-byte flag after 120 payload bytes.  wave64 layout: the low
+ * 32 bits of the flag after the 60 payload bytes of each 64-byte sector. */
+static void put_flag(uint8_t *line, uint64_t f, int layout) {
+    if (layout == LAYOUT_PAIR) {
+        for (int i = 0; i < 8; ++i) line[120 + i] = (uint8_t)(f >> (8 * i));
+    } else {
+        for (int i = 0; i < 4; ++i) line[60 + i] = line[124 + i] = (uint8_t)(f >> (8 * i));
+    }
 }
-static uint64_t get_flag(const uint8_t *line) {
-    uint64_t f = 0;
-    for (int i = 0; i < 8; ++i) f |= (uint64_t)line[120 + i] << (8 * i);
-    return f;
+static int flag_ok(const uint8_t *line, uint64_t want, int layout) {
+    if (layout == LAYOUT_PAIR) {
+        uint64_t f = 0;
+        for (int i = 0; i < 8; ++i) f |= (uint64_t)line[120 + i] << (8 * i);
+        return f == want;
+    }
+    uint32_t a = 0, b = 0;
+    for (int i = 0; i < 4; ++i) {
+        a |= (uint32_t)line[60 + i] << (8 * i);
+        b |= (uint32_t)line[124 + i] << (8 * i);
+    }
+    return a == (uint32_t)want && b == (uint32_t)want;
 }
 
 void ref_pack(const uint8_t *raw, size_t n, uint64_t flag_base, uint64_t flag_stride,
@@ -65,11 +79,14 @@ void ref_pack(const uint8_t *raw, size_t n, uint64_t flag_base, uint64_t flag_st
                 take(raw, n, base + 120, 8, line + 112);
             }
         } else {
-            size_t base = (L / 8) * 960, j = L % 8;
-            take(raw, n, base + 112 * j, 112, line);
-            take(raw, n, base + 896 + 8 * j, 8, line + 112);
+            size_t base = (L / 8) * 960;
+            for (size_t h = 0; h < 2; ++h) {           /* the line's two sectors */
+                size_t i = (L % 8) * 2 + h;
+                take(raw, n, base + 48 * i, 48, line + 64 * h);
+                take(raw, n, base + 768 + 12 * i, 12, line + 64 * h + 48);
+            }
         }
-        put_flag(line, flag_base + L * flag_stride);
+        put_flag(line, flag_base + L * flag_stride, layout);
     }
 }
 
@@ -78,7 +95,7 @@ size_t ref_unpack(const uint8_t *msg, size_t n, uint64_t flag_base, uint64_t fla
     size_t lines = ref_line_count(n, layout), bad = 0;
     for (size_t L = 0; L < lines; ++L) {
         const uint8_t *line = msg + L * 128;
-        if (get_flag(line) != flag_base + L * flag_stride) ++bad;
+        if (!flag_ok(line, flag_base + L * flag_stride, layout)) ++bad;
         if (layout == LAYOUT_PAIR) {
             size_t base = (L / 2) * 240;
             if (L % 2 == 0) {
@@ -88,9 +105,12 @@ size_t ref_unpack(const uint8_t *msg, size_t n, uint64_t flag_base, uint64_t fla
                 give(raw, n, base + 120, 8, line + 112);
             }
         } else {
-            size_t base = (L / 8) * 960, j = L % 8;
-            give(raw, n, base + 112 * j, 112, line);
-            give(raw, n, base + 896 + 8 * j, 8, line + 112);
+            size_t base = (L / 8) * 960;
+            for (size_t h = 0; h < 2; ++h) {
+                size_t i = (L % 8) * 2 + h;
+                give(raw, n, base + 48 * i, 48, line + 64 * h);
+                give(raw, n, base + 768 + 12 * i, 12, line + 64 * h + 48);
+            }
         }
     }
     return bad;

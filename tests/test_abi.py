@@ -1,0 +1,150 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header
+declares, agrees with the ctypes mirror on the descriptor layout, and its host
+side validation (no kernel launch involved) returns the documented errors."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from mintccl_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mintccl.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mint_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = declared_functions()
+    assert len(names) >= 12
+    L = _lib.lib()
+    for n in names:
+        assert hasattr(L, n), f"{n} not exported by libmintccl.so"
+        assert n in _lib.SYMBOLS, f"{n} has no ctypes signature"
+    assert set(_lib.SYMBOLS) == set(names)
+
+
+def test_version_and_strerror():
+    L = _lib.lib()
+    assert L.mint_version() >= 100
+    assert L.mint_strerror(0) == b"ok"
+    for code in range(-6, 0):
+        assert L.mint_strerror(code) not in (b"ok", b"unknown error")
+    assert L.mint_strerror(-99) == b"unknown error"
+
+
+def test_descriptor_layout_matches_the_header(tmp_path):
+    fields = [f for f, _ in _lib.RingOp._fields_]
+    src = tmp_path / "layout.c"
+    lines = ["#include <stdio.h>", "#include <stddef.h>", f'#include "{HEADER}"',
+             "int main(void){", '  printf("%zu\\n", sizeof(mint_ring_op));']
+    for f in fields:
+        lines.append(f'  printf("%zu\\n", offsetof(mint_ring_op, {f}));')
+    lines += ["  return 0;", "}"]
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c11", "-o", str(exe), str(src)])
+    out = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert out[0] == ctypes.sizeof(_lib.RingOp)
+    for f, off in zip(fields, out[1:]):
+        assert getattr(_lib.RingOp, f).offset == off, f
+
+
+def test_packed_bytes():
+    L = _lib.lib()
+    assert L.mint_ll128_packed_bytes(0, 0) == 0
+    assert L.mint_ll128_packed_bytes(120, 0) == 128
+    assert L.mint_ll128_packed_bytes(121, 0) == 256
+    assert L.mint_ll128_packed_bytes(1 << 20, 0) == 8739 * 128
+    assert L.mint_ll128_packed_bytes(1, 1) == 1024
+    assert L.mint_ll128_packed_bytes(960, 1) == 1024
+    assert L.mint_ll128_packed_bytes(961, 1) == 2048
+
+
+def make_op(**kw):
+    d = _lib.RingOp()
+    d.op, d.protocol, d.dtype, d.world = _lib.OP_REDUCESCATTER, _lib.PROTO_LL128, _lib.F16, 8
+    for i in range(9):
+        d.ring[i] = i % 8
+    for r in range(8):
+        d.input[r] = d.output[r] = 0x10000000 + r * 0x1000000
+        d.staging[r] = 0x70000000 + r * 0x1000000
+    d.count_bytes, d.row_stride = 1 << 20, 1 << 20
+    d.slot_bytes, d.nslots = 512 << 10, 8
+    d.waves_per_channel_group, d.threads_per_block = 16, 256
+    d.flag_epoch, d.status = 1, 0x60000000
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_plan_geometry_without_a_gpu():
+    L = _lib.lib()
+    d = make_op()
+    # 8 pipelines x 9 positions x (16 waves / 4 per block)
+    assert L.mint_ring_grid_blocks(d) == 8 * 9 * 4
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256
+    assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES)) == 8 * 8 * 4
+    d = make_op(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    d = make_op(op=_lib.OP_REDUCE, waves_per_channel_group=128, root=3)
+    assert L.mint_ring_grid_blocks(d) == 9 * 32
+
+
+@pytest.mark.parametrize("kw,err", [
+    (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
+    (dict(op=7), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(dtype=_lib.BYTES), _lib.ERR_ARG),          # a reduction needs a real dtype
+    (dict(flag_epoch=0), _lib.ERR_ARG), (dict(status=0), _lib.ERR_ARG),
+    (dict(threads_per_block=100), _lib.ERR_ARG),
+    (dict(slot_bytes=(512 << 10) + 512), _lib.ERR_GEOMETRY),
+    (dict(slot_bytes=4096), _lib.ERR_GEOMETRY),        # less than one block per pipeline
+    (dict(waves_per_channel_group=7), _lib.ERR_GEOMETRY),
+    (dict(nslots=0), _lib.ERR_GEOMETRY),
+    (dict(row_stride=(1 << 20) + 8), _lib.ERR_ALIGN),
+    (dict(row_stride=1 << 19), _lib.ERR_ALIGN),       # rows would overlap
+    (dict(count_bytes=(1 << 20) + 1, row_stride=1 << 21), _lib.ERR_ARG),
+    (dict(slot_bytes=1 << 30, nslots=8), _lib.ERR_TOO_LARGE),
+])
+def test_plan_rejects_bad_descriptors(kw, err):
+    assert _lib.lib().mint_ring_grid_blocks(make_op(**kw)) == err
+
+
+def test_plan_rejects_bad_buffers_and_rings():
+    L = _lib.lib()
+    d = make_op()
+    d.input[3] = 0
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+    d = make_op()
+    d.staging[2] += 8
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ALIGN
+    d = make_op()
+    d.ring[8] = 1                                    # ring does not close
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+    d = make_op()
+    d.ring[3] = 2                                    # rank 2 twice
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    code = ("import mintccl_amd._lib as l; l.SO_PATH=%r; l._lib=None\n"
+            "try:\n    l.lib()\nexcept RuntimeError as e:\n    print('RAISED', 'no CPU fallback' in str(e))\n"
+            % str(tmp_path / "nope.so"))
+    out = subprocess.check_output([sys.executable, "-c", code], cwd=ROOT).decode()
+    assert "RAISED True" in out
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "mintccl_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"

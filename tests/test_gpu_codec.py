@@ -1,0 +1,141 @@
+"""GPU parity, through the C ABI: copy, LL128 codec, element sum vs the oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ll128, ring
+from tests.helpers import as_bytes, random_bits, special_values_f16, uniform
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 15, 16, 17, 119, 120, 121, 240, 241, 959, 960, 961, 4096, 65536 + 2,
+         960 * 1000 + 8, (1 << 20) + 7]
+
+
+def dev_bytes(a: np.ndarray, dev) -> torch.Tensor:
+    return torch.from_numpy(a.copy()).to(dev)
+
+
+def test_device_is_mi355x_shaped(lib):
+    cu, xcd, wave = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.mint_device_info(cu, xcd, wave) == 0
+    assert wave.value == 64 and cu.value > 0 and xcd.value >= 1
+
+
+def test_blocks_are_dealt_round_robin_over_xcds(lib, dev):
+    from mintccl_amd import primitive
+    cu, xcd, wave = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    lib.mint_device_info(cu, xcd, wave)
+    m = primitive.xcd_map(64, dev).cpu().tolist()
+    assert m == [i % xcd.value for i in range(64)]
+
+
+@pytest.mark.parametrize("n", [0, 1, 16, 1000, (1 << 20) + 5, (64 << 20) + 16])
+def test_copy_simple(dev, n):
+    from mintccl_amd import primitive
+    g = torch.Generator().manual_seed(n)
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g).to(dev)
+    dst = torch.zeros(n + 64, dtype=torch.uint8, device=dev)
+    primitive.copy128(src, dst[:n])
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:n], src) and int(dst[n:].sum()) == 0
+
+
+@pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
+@pytest.mark.parametrize("n", SIZES)
+def test_pack_unpack_match_oracle(dev, layout, n):
+    from mintccl_amd import protocol
+    raw = np.random.default_rng(n).integers(0, 256, n, dtype=np.uint8)
+    d_raw = dev_bytes(raw, dev)
+    base = 3 + n
+    want = ll128.pack(raw, base, layout)
+    msg = torch.full((want.size + 256,), 0xEE, dtype=torch.uint8, device=dev)
+    protocol.pack(d_raw, base, layout, out=msg)
+    torch.cuda.synchronize()
+    got = msg.cpu().numpy()
+    assert (got[:want.size] == want).all()
+    assert (got[want.size:] == 0xEE).all()            # nothing written past the end
+    out = torch.full((n + 64,), 0xEE, dtype=torch.uint8, device=dev)
+    bad = torch.zeros(1, dtype=torch.int64, device=dev)
+    if n:
+        protocol.unpack(msg, out[:n], base, layout, bad_flags=bad)
+    torch.cuda.synchronize()
+    assert (out.cpu().numpy()[:n] == raw).all() and (out.cpu().numpy()[n:] == 0xEE).all()
+    assert bad.item() == 0
+
+
+@pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
+def test_unpack_counts_wrong_flags(dev, layout):
+    from mintccl_amd import protocol
+    raw = np.arange(20000, dtype=np.uint8)
+    msg = ll128.pack(raw, 1, layout)
+    msg[5 * 128 + (121 if layout == ll128.LAYOUT_PAIR else 61)] ^= 4
+    msg[17 * 128 + 127] ^= 1
+    d_msg = dev_bytes(msg, dev)
+    out = torch.zeros(raw.size, dtype=torch.uint8, device=dev)
+    bad = torch.zeros(1, dtype=torch.int64, device=dev)
+    protocol.unpack(d_msg, out, 1, layout, bad_flags=bad)
+    torch.cuda.synchronize()
+    assert bad.item() == 2 == ll128.unpack(msg, raw.size, 1, layout)[1]
+
+
+@pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
+@pytest.mark.parametrize("stride", [1, 0])
+def test_config1_roundtrip_on_device(dev, layout, stride):
+    # BASELINE config 1 on the GPU: 1 MiB fp16 uniform[-1,1] seed 0
+    from mintccl_amd import protocol
+    x = uniform(524288, -1.0, 1.0, 0)
+    d = x.to(dev)
+    msg = protocol.pack(d, 1, layout, flag_stride=stride)
+    want = ll128.pack(as_bytes(x), 1, layout, flag_stride=stride)
+    assert (msg.cpu().numpy() == want).all()
+    back = torch.empty_like(d)
+    bad = torch.zeros(1, dtype=torch.int64, device=dev)
+    protocol.unpack(msg, back, 1, layout, flag_stride=stride, bad_flags=bad)
+    assert torch.equal(back.view(torch.int16), d.view(torch.int16)) and bad.item() == 0
+
+
+@pytest.mark.parametrize("dt,tdt,bits", [("f16", torch.float16, 16), ("bf16", torch.bfloat16, 16),
+                                         ("f32", torch.float32, 32)])
+@pytest.mark.parametrize("n", [1, 7, 8, 100003, 1 << 20])
+def test_elementwise_sum_random_bit_patterns(dev, dt, tdt, bits, n):
+    from mintccl_amd import primitive
+    a, b = random_bits(n, bits, n + 1), random_bits(n, bits, n + 2)
+    iv, nv = (torch.int32, np.int32) if bits == 32 else (torch.int16, np.int16)
+    ta = torch.from_numpy(a.view(nv)).to(dev).view(tdt)
+    tb = torch.from_numpy(b.view(nv)).to(dev).view(tdt)
+    got = primitive.Sum(ta, tb).view(iv).cpu().numpy()
+    want = ring.add_rn(a, b, dt)
+    assert ring.same_values(got, want, dt)
+    if dt != "f16":       # bf16 canonicalises NaN, f32 NaNs aside: bits must agree
+        w = want.view(np.uint16 if bits == 16 else np.uint32)
+        g = got.view(np.uint16 if bits == 16 else np.uint32)
+        nan = np.isnan(ring.to_float64(want, dt))
+        assert (g[~nan] == w[~nan]).all()
+
+
+def test_elementwise_sum_f16_special_values_and_subnormals(dev):
+    from mintccl_amd import primitive
+    sp = np.concatenate([special_values_f16(), np.arange(0, 1100, dtype=np.uint16),
+                         np.arange(0x8000, 0x8000 + 1100, dtype=np.uint16)])
+    aa, bb = np.meshgrid(sp, sp)
+    aa, bb = aa.reshape(-1).copy(), bb.reshape(-1).copy()
+    ta = torch.from_numpy(aa.view(np.int16)).to(dev).view(torch.float16)
+    tb = torch.from_numpy(bb.view(np.int16)).to(dev).view(torch.float16)
+    got = primitive.SumFP16(ta, tb).view(torch.int16).cpu().numpy()
+    want = ring.add_rn(aa, bb, "f16")
+    assert ring.same_values(got, want, "f16")
+    finite = ~np.isnan(ring.to_float64(want, "f16"))
+    assert (got.view(np.uint16)[finite] == want.view(np.uint16)[finite]).all()   # -0, subnormals
+
+
+def test_alignment_is_rejected_not_faulted(lib, dev):
+    from mintccl_amd import _lib
+    buf = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    p = buf.data_ptr()
+    assert lib.mint_copy_simple(p + 1, p + 2048, 64, 0, 0, 0) == _lib.ERR_ALIGN
+    assert lib.mint_ll128_pack(p + 8, p + 2048, 64, 1, 1, 0, 0) == _lib.ERR_ALIGN
+    assert lib.mint_ll128_pack(p, p + 2048, 64, 1, 1, 5, 0) == _lib.ERR_ARG
+    assert lib.mint_elementwise_sum(p, p + 4, p + 2048, 8, 0, 0) == _lib.ERR_ALIGN

@@ -1,0 +1,310 @@
+"""GPU parity of the ring collectives against the oracle, through the
+operator surface and the C ABI (bit-exact: payloads for the copying ops,
+reference fold order for the reductions)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ring
+from tests.helpers import TORCH_DT, as_bytes, normal, rank_rows, uniform
+
+pytestmark = pytest.mark.gpu
+
+
+def make_comm(world, **kw):
+    from mintccl_amd.common import VirtualComm
+    kw.setdefault("spin_budget", 400000)      # ~ a second: a lost line fails, never hangs
+    return VirtualComm(world_size=world, **kw)
+
+
+def run_reducescatter(comm, bufs):
+    from mintccl_amd.reducescatter import reducescatter
+    comm.run(lambda r: reducescatter(bufs[r], comm))
+    comm.check()
+
+
+def run_allgather(comm, bufs):
+    from mintccl_amd.allgather import allgather
+    comm.run(lambda r: allgather(bufs[r], comm))
+    comm.check()
+
+
+def run_reduce(comm, bufs, root):
+    from mintccl_amd.reduce import reduce
+    comm.run(lambda r: reduce(bufs[r], root, comm))
+    comm.check()
+
+
+def run_broadcast(comm, bufs, root):
+    from mintccl_amd.broadcast import broadcast
+    comm.run(lambda r: broadcast(bufs[r], root, comm))
+    comm.check()
+
+
+def same(bufs, want) -> bool:
+    return all(np.array_equal(as_bytes(b), w) for b, w in zip(bufs, want))
+
+
+WORLDS = [2, 3, 5, 8]
+ROW_ELEMS = [1, 8, 479, 480, 481, 4096, 100003]      # ragged, one block, many steps
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("n", ROW_ELEMS)
+def test_reducescatter_f16(dev, world, n):
+    if (n * 2) % 16:                 # rows of a (world, n) buffer must start 16-byte aligned
+        n = (n + 7) // 8 * 8
+    host = rank_rows(world, n, "f16")
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, buff_size_=world * 8 * 8192, nslots=8, waves_per_rank=8 * world)
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("proto", [0, 1])
+@pytest.mark.parametrize("place", [0, 1])
+def test_reducescatter_dtypes_protocols_placements(dev, dt, proto, place):
+    world, n = 8, 65536 + 8
+    host = rank_rows(world, n, dt)
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, protocol=proto, placement=place)
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], dt))
+
+
+def test_reducescatter_special_values(dev):
+    # overflow to inf, inf - inf, subnormals, signed zeros ride the ring unharmed
+    world, n = 4, 960
+    vals = torch.tensor([65504.0, -65504.0, 6e-8, -6e-8, 0.0, -0.0, float("inf"), float("-inf"),
+                         1.0, 2048.0, 1e-4, 3.0], dtype=torch.float16)
+    g = torch.Generator().manual_seed(5)
+    host = [vals[torch.randint(0, len(vals), (world * n,), generator=g)].reshape(world, n)
+            for _ in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    run_reducescatter(comm, bufs)
+    want = ring.reducescatter([as_bytes(h) for h in host], "f16")
+    for b, w in zip(bufs, want):
+        assert ring.same_values(as_bytes(b), w, "f16")
+
+
+def test_reducescatter_order_is_the_reference_ring_order(dev):
+    # binary16 has ulp 2 at 2048, so 2048 + 1 ties back to 2048 while
+    # (1 + 1) + 2048 = 2050: where the large value enters the fold is visible.
+    # rows[r][c] = rank r's value for chunk c; chunk c folds in the order
+    # c, c+1, ... (7_reducescatter.py:54-73), starting from rank c's own value.
+    world, n = 4, 8
+    rows = [[2048.0, 1.0, 2048.0, 1.0], [1.0, 1.0, 1.0, 1.0], [1.0, 2048.0, 1.0, 2048.0],
+            [1.0, 1.0, 1.0, 1.0]]
+    host = [torch.tensor(rows[r], dtype=torch.float16).repeat_interleave(n).reshape(world, n).contiguous()
+            for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    run_reducescatter(comm, bufs)
+    got = [float(bufs[c][c, 0]) for c in range(world)]
+    assert got[0] == 2048.0   # 2048, +1 -> 2048, +1 -> 2048, +1 -> 2048
+    assert got[1] == 2048.0   # order 1,2,3,0: 1, +2048 -> 2048, +1, +1 (unrotated 0,1,2,3 gives 2052)
+    assert got[2] == 2052.0   # order 2,3,0,1: 1, 2, 2050, 2051 -> 2052 (owner-last order gives 2048)
+    assert got[3] == 2052.0   # order 3,0,1,2: 1, 2, 3, 2051 -> 2052 (reverse order gives 2048)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("root", [0, 1])
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_reduce(dev, world, root, dt):
+    n = 70001
+    host = [normal(n, 3000 + r, TORCH_DT[dt]) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    run_reduce(comm, bufs, root)
+    assert same(bufs, ring.reduce([as_bytes(h) for h in host], root, dt))
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("nbytes", [1, 7, 960, 961, 1 << 20, (1 << 20) + 3])
+@pytest.mark.parametrize("proto", [0, 1])
+def test_broadcast_bytes(dev, world, nbytes, proto):
+    root = world - 1
+    g = torch.Generator().manual_seed(nbytes)
+    host = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g) for _ in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, protocol=proto)
+    run_broadcast(comm, bufs, root)
+    for b in bufs:
+        assert torch.equal(b.cpu(), host[root])
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("n", [8, 480, 488, 65536])
+@pytest.mark.parametrize("proto", [0, 1])
+def test_allgather(dev, world, n, proto):
+    host = [uniform(world * n, -1.0, 1.0, 4 + r).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, protocol=proto)
+    run_allgather(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+
+
+def test_permuted_ring(dev):
+    # a non-uniform topology whose best ring is not the identity
+    from mintccl_amd.topology import find_ring
+    world, n = 4, 5000
+    fast, slow = 50.0, 5.0
+    edges = {(0, 2): fast, (2, 1): fast, (1, 3): fast, (3, 0): fast, (0, 1): slow, (2, 3): slow}
+    topo = {i: [] for i in range(world)}
+    for (a, b), bw in edges.items():
+        topo[a].append((b, bw))
+        topo[b].append((a, bw))
+    ring_ = find_ring(topo)
+    assert ring_ in ([0, 2, 1, 3, 0], [0, 3, 1, 2, 0])
+    host = rank_rows(world, n + (-n) % 8, "f16")
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    comm.topology = topo
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16", ring_))
+    host2 = [normal(3001, 50 + r) for r in range(world)]
+    bufs2 = [h.to(dev) for h in host2]
+    run_reduce(comm, bufs2, 1)
+    assert same(bufs2, ring.reduce([as_bytes(h) for h in host2], 1, "f16", ring_))
+
+
+def test_many_launches_reuse_staging_without_clearing(dev):
+    # flags carry a per-launch epoch: stale lines of earlier launches, of other
+    # sizes and other collectives, are never mistaken for data
+    world = 8
+    comm = make_comm(world)
+    for i, n in enumerate([4096, 480, 100000, 8, 4096, 52000]):
+        host = rank_rows(world, n, "f16", seed0=100 * i)
+        bufs = [h.to(dev) for h in host]
+        run_reducescatter(comm, bufs)
+        assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+        host = [uniform(world * n, -1.0, 1.0, i + r).reshape(world, n) for r in range(world)]
+        bufs = [h.to(dev) for h in host]
+        run_allgather(comm, bufs)
+        assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+
+
+def test_a_lost_producer_times_out_instead_of_hanging(dev):
+    from mintccl_amd import _lib
+    from mintccl_amd.common import RingTimeout
+    world, n = 4, 4096
+    comm = make_comm(world, spin_budget=2000)
+    bufs = [torch.zeros(n, dtype=torch.float16, device=dev) for _ in range(world)]
+    d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n * 2, {0: bufs[0].data_ptr()},
+                     {r: bufs[r].data_ptr() for r in range(1, world)}, [0, 1, 2, 3, 0],
+                     root=0, skip_origin=True)
+    comm.launch(d)
+    with pytest.raises(RingTimeout):
+        comm.check()
+    # the communicator is usable afterwards
+    host = [normal(n, r) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    run_broadcast(comm, bufs, 2)
+    for b in bufs:
+        assert torch.equal(b.cpu(), host[2])
+
+
+def test_residency_is_checked(dev):
+    from mintccl_amd import _lib
+    world = 8
+    comm = make_comm(world, buff_size_=64 << 20, nslots=8, waves_per_rank=8192)
+    bufs = [torch.zeros(world, 4096, dtype=torch.float16, device=dev) for _ in range(world)]
+    from mintccl_amd.reducescatter import reducescatter
+    with pytest.raises(_lib.MintError) as e:
+        comm.run(lambda r: reducescatter(bufs[r], comm))
+    assert e.value.code == _lib.ERR_RESIDENCY
+
+
+def run_probe(lib, dev, pairs, iters, cp, place, per_sector):
+    st = torch.zeros(pairs * (4 * 1024 + 128), dtype=torch.uint8, device=dev)
+    cnt = torch.zeros(8, dtype=torch.int64, device=dev)
+    assert lib.mint_torn_line_probe(st.data_ptr(), st.numel(), pairs, iters, cp, place, per_sector,
+                                    3, 400000, cnt.data_ptr(), 0) == 0
+    torch.cuda.synchronize()
+    return cnt.cpu().tolist()
+
+
+@pytest.mark.parametrize("cp", [0, 1])
+@pytest.mark.parametrize("place", [0, 1])
+def test_no_torn_sectors(lib, dev, cp, place):
+    # every 64-byte sector carries its tag and a payload that is a function of
+    # the tag: once all 16 tags of a block are seen, every byte must belong
+    pairs, iters = 2048, 20000
+    checked, torn, polls, timeouts, first_half = run_probe(lib, dev, pairs, iters, cp, place, 1)[:5]
+    assert timeouts == 0 and checked == pairs * iters * 8
+    assert torn == 0
+
+
+def test_one_flag_per_128_byte_line_is_not_enough(lib, dev):
+    # the reference's assumption (protocol.py:31-35): whoever sees the flag in
+    # the last bytes of a 128-byte line has the whole line.  On this GPU the
+    # first 64-byte sector can still be the old one; whenever that is
+    # observed it is exactly that sector, never a finer tear.
+    pairs, iters = 2048, 20000
+    checked, torn, polls, timeouts, first_half = run_probe(lib, dev, pairs, iters, 0, 0, 0)[:5]
+    assert timeouts == 0 and checked == pairs * iters * 8
+    assert torn == first_half
+    print(f"lines checked {checked}, torn {torn} (first sector stale: {first_half})")
+
+
+# ---- BASELINE configurations at their full sizes ---------------------------
+def test_config3_broadcast_64mib_8_ranks(dev):
+    world, n = 8, 33554432
+    root_data = uniform(n, -4.0, 4.0, 2).to(dev)
+    bufs = [root_data.clone() if r == 0 else torch.zeros(n, dtype=torch.float16, device=dev)
+            for r in range(world)]
+    comm = make_comm(world, buff_size_=8 * 512 * 1024, nslots=8)
+    run_broadcast(comm, bufs, 0)
+    for b in bufs:
+        assert torch.equal(b.view(torch.int16), root_data.view(torch.int16))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_config4_reducescatter_and_reduce_32m_elements(dev, dt):
+    # 32 Mi elements per rank, seed 3000 + rank, 1 MiB slots.  Full-size check
+    # against the device adder folded in ring order (itself checked against the
+    # oracle above), plus the oracle on a slice of every chunk.
+    from mintccl_amd import primitive
+    world, n_total = 8, 33554432
+    n = n_total // world
+    bufs = [normal(n_total, 3000 + r, TORCH_DT[dt]).reshape(world, n).to(dev) for r in range(world)]
+    orig = [b.clone() for b in bufs]
+    comm = make_comm(world, buff_size_=8 << 20, nslots=8, waves_per_rank=256)
+    run_reducescatter(comm, bufs)
+    for c in range(world):
+        acc = orig[c][c].clone()
+        for k in range(1, world):
+            acc = primitive.Sum(orig[(c + k) % world][c].contiguous(), acc)
+        assert torch.equal(bufs[c][c].view(torch.uint8), acc.view(torch.uint8))
+        for r in range(world):
+            if r != c:
+                assert torch.equal(bufs[r][c], orig[r][c])
+        sl = slice(n - 4099, n)
+        want = ring.fold([as_bytes(orig[r][c, sl]) for r in range(world)],
+                         ring.fold_order(ring.identity_ring(world), c), dt)
+        assert np.array_equal(as_bytes(bufs[c][c, sl]), want)
+    flat = [o.reshape(-1).clone() for o in orig]
+    run_reduce(comm, flat, 0)
+    acc = orig[0].reshape(-1).clone()
+    for k in range(1, world):
+        acc = primitive.Sum(orig[k].reshape(-1), acc)
+    assert torch.equal(flat[0].view(torch.uint8), acc.view(torch.uint8))
+
+
+def test_headline_reducescatter_256mib_fp16(dev):
+    from mintccl_amd import primitive
+    world, n_total = 8, 134217728
+    n = n_total // world
+    g = torch.Generator(device=dev).manual_seed(7)
+    bufs = [torch.randn(world, n, generator=g, device=dev, dtype=torch.float16) for _ in range(world)]
+    orig = [b.clone() for b in bufs]
+    comm = make_comm(world)
+    run_reducescatter(comm, bufs)
+    for c in range(world):
+        acc = orig[c][c].clone()
+        for k in range(1, world):
+            acc = primitive.Sum(orig[(c + k) % world][c].contiguous(), acc)
+        assert torch.equal(bufs[c][c].view(torch.int16), acc.view(torch.int16))

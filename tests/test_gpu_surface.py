@@ -1,0 +1,158 @@
+"""The reference-named operator surface: send / recv / sync, argument checks,
+asynchronous launch, BASELINE config 2 and the allgather sweep of config 5."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import as_bytes, normal, uniform
+
+pytestmark = pytest.mark.gpu
+
+
+def make_comm(world, **kw):
+    from mintccl_amd.common import VirtualComm
+    kw.setdefault("spin_budget", 400000)
+    return VirtualComm(world_size=world, **kw)
+
+
+@pytest.mark.parametrize("nbytes", [2, 4096, (1 << 20) + 6])
+def test_direct_send_recv(dev, nbytes):
+    from mintccl_amd import sendrecv_direct as m
+    comm = make_comm(2)
+    src = normal(nbytes // 2, 1).to(dev)
+    dst = torch.zeros_like(src)
+    with comm.rank(0):
+        m.send(src, 1, comm)
+    with comm.rank(1):
+        m.recv(dst, 0, comm=comm)
+    assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+
+
+@pytest.mark.parametrize("module", ["sendrecv_buffer", "sendrecv_indirect"])
+@pytest.mark.parametrize("route", [None, [0, 2, 1], [0, 3, 2, 1]])
+@pytest.mark.parametrize("n", [1, 123457])
+def test_deferred_send_recv_sync(dev, module, route, n):
+    import importlib
+    m = importlib.import_module(f"mintccl_amd.{module}")
+    comm = make_comm(4)
+    src = torch.randn(n, generator=torch.Generator().manual_seed(n)).to(dev)   # fp32 like the reference test
+    dst = torch.zeros_like(src)
+    with comm.rank(0):
+        m.send(src, 1, comm)
+    with comm.rank(1):
+        m.recv(dst, 0, comm)
+    for r in range(4):                      # everyone calls sync (3_sendrecv_buffer.py:98)
+        with comm.rank(r):
+            m.sync(comm, route=route)
+    comm.check()
+    assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
+
+
+def test_sync_rejects_mismatched_pairs(dev):
+    from mintccl_amd import sendrecv_buffer as m
+    comm = make_comm(2)
+    a = torch.zeros(16, device=dev)
+    b = torch.zeros(32, device=dev)
+    with comm.rank(0):
+        m.send(a, 1, comm)
+    with comm.rank(1):
+        m.recv(b, 0, comm)
+    with pytest.raises(ValueError):
+        m.sync(comm)
+
+
+def test_config2_sendrecv_256mib_ll128_and_simple(dev):
+    # 134,217,728 fp16 normal(0,1) seed 1, rank 0 -> rank 1, 512 KiB slots
+    from mintccl_amd import sendrecv_buffer as m, sendrecv_direct as direct
+    src = normal(134217728, 1).to(dev)
+    for proto in (0, 1):
+        comm = make_comm(2, buff_size_=8 * 512 * 1024, nslots=8, protocol=proto)
+        dst = torch.zeros_like(src)
+        with comm.rank(0):
+            m.send(src, 1, comm)
+        with comm.rank(1):
+            m.recv(dst, 0, comm)
+        m.sync(comm)
+        comm.check()
+        assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+    comm = make_comm(2)
+    dst = torch.zeros_like(src)
+    with comm.rank(0):
+        direct.send(src, 1, comm)
+    with comm.rank(1):
+        direct.recv(dst, 0, comm=comm)
+    assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+
+
+@pytest.mark.parametrize("proto", [0, 1])
+def test_config5_allgather_sweep(dev, proto):
+    # per-rank shard 512 B .. 8 MiB here (the benchmark sweeps to 128 MiB),
+    # fixed 8 x 512 KiB staging
+    from mintccl_amd.allgather import allgather
+    world = 8
+    comm = make_comm(world, buff_size_=8 * 512 * 1024, nslots=8, protocol=proto)
+    for log2 in range(9, 24, 2):
+        n = (1 << log2) // 2
+        host = [uniform(world * n, -1.0, 1.0, 4 + r).reshape(world, n) for r in range(world)]
+        bufs = [h.to(dev) for h in host]
+        comm.run(lambda r: allgather(bufs[r], comm))
+        comm.check()
+        for r in range(world):
+            for c in range(world):
+                assert torch.equal(bufs[r][c].cpu(), host[c][c]), (log2, r, c)
+
+
+def test_argument_checks(dev):
+    from mintccl_amd.reduce import reduce
+    from mintccl_amd.reducescatter import reducescatter
+    comm = make_comm(2)
+    with comm.rank(0):
+        with pytest.raises(TypeError):
+            reduce(torch.zeros(8, dtype=torch.int32, device=dev), 0, comm)
+        with pytest.raises(TypeError):
+            reduce(torch.zeros(8, dtype=torch.float16), 0, comm)          # host tensor
+        with pytest.raises(ValueError):
+            reducescatter(torch.zeros(3, 3, dtype=torch.float16, device=dev), comm)
+        with pytest.raises(ValueError):
+            reduce(torch.zeros(8, 8, dtype=torch.float16, device=dev).t(), 0, comm)
+    with pytest.raises(RuntimeError):
+        comm.Get_rank()                                                   # outside a rank context
+    a = torch.zeros(8, dtype=torch.float16, device=dev)
+    b = torch.zeros(16, dtype=torch.float16, device=dev)
+    with comm.rank(0):
+        reduce(a, 0, comm)
+    with comm.rank(1):
+        with pytest.raises(ValueError):
+            reduce(b, 0, comm)                                            # ranks disagree on size
+
+
+def test_world_of_one_is_a_no_op(dev):
+    from mintccl_amd.reducescatter import reducescatter
+    from mintccl_amd.broadcast import broadcast
+    comm = make_comm(1)
+    x = normal(4096, 0).to(dev).reshape(1, -1)
+    y = x.clone()
+    with comm.rank(0):
+        reducescatter(x, comm)
+        broadcast(x, 0, comm)
+    comm.check()
+    assert torch.equal(x, y)
+
+
+def test_launch_is_asynchronous_and_stream_ordered(dev):
+    # the operator enqueues on the current stream and returns; a later kernel
+    # on the same stream sees the result
+    from mintccl_amd.broadcast import broadcast
+    world, n = 8, 1 << 22
+    comm = make_comm(world)
+    s = torch.cuda.Stream(device=dev)
+    host = uniform(n, -4.0, 4.0, 9)
+    with torch.cuda.stream(s):
+        bufs = [host.to(dev, non_blocking=False) if r == 3 else
+                torch.zeros(n, dtype=torch.float16, device=dev) for r in range(world)]
+        comm.run(lambda r: broadcast(bufs[r], 3, comm))
+        total = torch.stack([b.float().sum() for b in bufs])
+    s.synchronize()
+    comm.check()
+    want = host.to(dev).float().sum()
+    assert torch.all(total == want)

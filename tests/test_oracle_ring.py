@@ -1,0 +1,195 @@
+"""Pins oracle/ring.py: the element addition and the ring fold order."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, ll128, ring
+from tests.helpers import random_bits, special_values_f16
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def exact_then_round_once_f16(a_bits, b_bits):
+    """binary64 holds the sum of two binary16 values exactly; one rounding."""
+    a = a_bits.view(np.float16).astype(np.float64)
+    b = b_bits.view(np.float16).astype(np.float64)
+    with np.errstate(all="ignore"):
+        return (a + b).astype(np.float16).view(np.uint16)
+
+
+def exact_then_round_once_bf16(a_bits, b_bits):
+    a = (a_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    b = (b_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    with np.errstate(all="ignore"):
+        s = a + b                      # exact unless exponents are > 52 apart,
+    # in which case the smaller operand is below half an ulp of bf16 anyway
+    # round binary64 -> bf16 (8 significant bits, emin -126) to nearest even
+    # with frexp / rint, then read the bits off the (exactly representable) value
+    with np.errstate(all="ignore"):
+        m, e = np.frexp(s)                                   # s = m * 2**e, 0.5 <= |m| < 1
+        e = np.maximum(e, -125)                              # subnormal quantum 2**-133
+        q = np.ldexp(np.rint(np.ldexp(s, 8 - e)), e - 8)     # rint: ties to even
+        q32 = q.astype(np.float32)                           # exact, or overflow to inf
+    out = (q32.view(np.uint32) >> 16).astype(np.uint16)
+    big = np.abs(q) >= 2.0 ** 128
+    out[big] = np.where(q[big] > 0, 0x7F80, 0xFF80).astype(np.uint16)
+    out[np.isnan(s)] = 0x7FC0
+    return out
+
+
+def test_add_f16_is_one_correct_rounding():
+    a, b = random_bits(400000, 16, 1), random_bits(400000, 16, 2)
+    got = ring.add_rn(a, b, "f16").view(np.uint16)
+    want = exact_then_round_once_f16(a, b)
+    assert ring.same_values(got, want, "f16")
+
+
+def test_add_bf16_is_one_correct_rounding():
+    a, b = random_bits(400000, 16, 3), random_bits(400000, 16, 4)
+    got = ring.add_rn(a, b, "bf16").view(np.uint16)
+    want = exact_then_round_once_bf16(a, b)
+    assert ring.same_values(got, want, "bf16")
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_add_matches_integer_softfloat(dt):
+    a, b = random_bits(1 << 20, 16, 5), random_bits(1 << 20, 16, 6)
+    assert ring.same_values(ring.add_rn(a, b, dt), cref.add(a, b, dt), dt)
+    sp = special_values_f16()
+    aa, bb = np.meshgrid(sp, sp)
+    aa, bb = aa.reshape(-1).copy(), bb.reshape(-1).copy()
+    assert ring.same_values(ring.add_rn(aa, bb, dt), cref.add(aa, bb, dt), dt)
+
+
+def test_add_f16_exhaustive_near_subnormals():
+    # every pair of the 2048 smallest magnitudes of both signs: subnormal
+    # results, cancellation to +0, -0 + -0 = -0
+    mags = np.arange(0, 1100, dtype=np.uint16)
+    vals = np.concatenate([mags, mags | 0x8000])
+    aa, bb = np.meshgrid(vals, vals)
+    aa, bb = aa.reshape(-1).copy(), bb.reshape(-1).copy()
+    got = ring.add_rn(aa, bb, "f16").view(np.uint16)
+    assert (got == cref.add(aa, bb, "f16").view(np.uint16)).all()
+    assert (got == exact_then_round_once_f16(aa, bb)).all()
+
+
+@pytest.mark.parametrize("dt,tdt", [("f16", torch.float16), ("bf16", torch.bfloat16),
+                                    ("f32", torch.float32)])
+def test_add_matches_torch_cpu(dt, tdt):
+    bits = 32 if dt == "f32" else 16
+    a, b = random_bits(200000, bits, 7), random_bits(200000, bits, 8)
+    iv = torch.int32 if bits == 32 else torch.int16
+    ta = torch.from_numpy(a.view(np.int32 if bits == 32 else np.int16)).view(tdt)
+    tb = torch.from_numpy(b.view(np.int32 if bits == 32 else np.int16)).view(tdt)
+    want = (ta + tb).view(iv).numpy()
+    assert ring.same_values(ring.add_rn(a, b, dt), want, dt)
+
+
+def test_hand_computed_fold_order():
+    # 2048 has ulp 2 in binary16: 2048 + 1 -> 2048 (tie to even), so the
+    # position of the large value in the fold is visible in the result
+    f = lambda *v: [np.array([x], dtype=np.float16).view(np.uint8) for x in v]
+    rows = f(2048.0, 1.0, 1.0)
+    as_f = lambda raw: float(raw.view(np.float16)[0])
+    assert as_f(ring.fold(rows, [0, 1, 2], "f16")) == 2048.0   # (2048+1)+1
+    assert as_f(ring.fold(rows, [1, 2, 0], "f16")) == 2050.0   # (1+1)+2048
+
+
+def test_hand_computed_fold_order_exact_values():
+    f = lambda *v: [np.array([x], dtype=np.float16).view(np.uint8) for x in v]
+    as_f = lambda raw: float(raw.view(np.float16)[0])
+    rows = f(2048.0, 1.0, 1.0)
+    # acc = 1; 2048 + 1 = 2049 -> 2048; 1 + 2048 = 2049 -> 2048
+    assert as_f(ring.fold(rows, [2, 0, 1], "f16")) == 2048.0
+
+
+def test_reduce_order_follows_ring_from_root():
+    with open(os.path.join(GOLD, "fold_vectors.json")) as f:
+        gold = json.load(f)
+    # element 0 by hand: root 0 -> ((2048+1)+1)+0.5 = 2048; root 1 -> ((1+1)+0.5)+2048 = 2050
+    by_root = {c["root"]: c for c in gold["cases"]}
+    assert np.array(by_root[0]["result_f16_bits"], dtype=np.uint16).view(np.float16)[0] == 2048.0
+    assert np.array(by_root[1]["result_f16_bits"], dtype=np.uint16).view(np.float16)[0] == 2050.0
+    for c in gold["cases"]:
+        xs = [np.array(r, dtype=np.uint16).view(np.uint8) for r in c["rows_f16_bits"]]
+        out = ring.reduce(xs, c["root"], "f16")
+        assert out[c["root"]].view(np.uint16).tolist() == c["result_f16_bits"]
+        for r in range(4):
+            if r != c["root"]:
+                assert (out[r] == xs[r]).all()       # non-roots keep their data
+
+
+def test_fold_order_with_a_permuted_ring():
+    ring_ = [0, 2, 1, 3, 0]
+    assert ring.fold_order(ring_, 1) == [1, 3, 0, 2]
+    assert ring.fold_order(ring_, 0) == [0, 2, 1, 3]
+    assert ring.fold_order(ring.identity_ring(8), 5) == [5, 6, 7, 0, 1, 2, 3, 4]
+
+
+def test_two_ranks_is_one_commutative_add():
+    a, b = random_bits(5000, 16, 11), random_bits(5000, 16, 12)
+    x = [a.view(np.uint8), b.view(np.uint8)]
+    r0 = ring.reduce(x, 0, "f16")[0]
+    r1 = ring.reduce(x, 1, "f16")[1]
+    assert ring.same_values(r0, r1, "f16")
+    assert ring.same_values(r0, ring.add_rn(a, b, "f16"), "f16")
+
+
+@pytest.mark.parametrize("dt", ring.DTYPES)
+def test_fold_stays_within_half_ulp_steps_of_exact_sum(dt):
+    n_ranks, n = 8, 4096
+    g = torch.Generator().manual_seed(1)
+    xs = [torch.randn(n, generator=g).to({"f16": torch.float16, "bf16": torch.bfloat16,
+                                          "f32": torch.float32}[dt]) for _ in range(n_ranks)]
+    raw = [x.view(torch.uint8).numpy() for x in xs]
+    got = ring.to_float64(ring.reduce(raw, 0, dt)[0], dt)
+    exact = sum(ring.to_float64(r, dt) for r in raw)
+    eps = {"f16": 2.0 ** -11, "bf16": 2.0 ** -8, "f32": 2.0 ** -24}[dt]
+    bound = (n_ranks - 1) * eps * sum(np.abs(ring.to_float64(r, dt)) for r in raw)
+    assert (np.abs(got - exact) <= bound + 1e-30).all()
+
+
+@pytest.mark.parametrize("dt", ring.DTYPES)
+@pytest.mark.parametrize("world", [2, 3, 8])
+def test_wire_walk_equals_closed_form(dt, world):
+    item = ring.ITEMSIZE[dt]
+    n = 1237
+    rng = np.random.default_rng(world)
+    tdt = {"f16": np.float16, "bf16": None, "f32": np.float32}[dt]
+
+    def rand(count):
+        v = rng.standard_normal(count).astype(np.float32)
+        if dt == "bf16":
+            return (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+        return v.astype(tdt).view(np.uint8)
+
+    xs = [rand(n) for _ in range(world)]
+    for layout in (ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64):
+        assert all((a == b).all() for a, b in zip(ring.reduce(xs, 1, dt),
+                                                  ring.reduce_wire(xs, 1, dt, layout=layout)))
+    rows = [rand(world * n) for _ in range(world)]
+    assert all((a == b).all() for a, b in zip(ring.reducescatter(rows, dt),
+                                              ring.reducescatter_wire(rows, dt)))
+    assert all((a == b).all() for a, b in zip(ring.broadcast(xs, world - 1),
+                                              ring.broadcast_wire(xs, world - 1)))
+    assert n * item == xs[0].size
+
+
+def test_copy_collectives_are_identities():
+    world, n = 4, 100
+    rng = np.random.default_rng(0)
+    rows = [rng.integers(0, 256, world * n, dtype=np.uint8) for _ in range(world)]
+    out = ring.allgather(rows)
+    for r in range(world):
+        for c in range(world):
+            assert (out[r].reshape(world, n)[c] == rows[c].reshape(world, n)[c]).all()
+    out = ring.sendrecv(rows, 2, 0)
+    assert (out[0] == rows[2]).all() and (out[1] == rows[1]).all()
+    rs = ring.reducescatter([r.view(np.uint8) for r in rows], "f16")
+    for r in range(world):
+        for c in range(world):
+            if r != c:      # only row r of rank r changes
+                assert (rs[r].reshape(world, n)[c] == rows[r].reshape(world, n)[c]).all()
