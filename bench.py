@@ -1,0 +1,172 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 8-virtual-rank LL128 ring reduce-scatter, fp16, 256 MiB
+per rank, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one fused launch that runs all 8 ranks' kernels over inputs that
+are already resident in HBM.  Prints ONE JSON line:
+
+  value     algorithmic payload bytes per step / wall time per step, GB/s.
+            Payload bytes = (3 N + 1) S: per chunk of S / N bytes, N reads of
+            the ranks' own rows, N staging writes, N staging reads, 1 output
+            write (S = 256 MiB per rank, N = 8 -> 6.711 GB).
+  roofline  the same bytes over the kernel's own duration (HIP events on the
+            launch stream), against the 8 TB/s HBM peak.  `traffic` is the HBM
+            bytes per launch measured with rocprofv3 counters
+            (profiles/reducescatter_ll128_f16_256mib_pmc.txt).
+  copy_*    measured HBM copy bandwidth of the library's own 16 B / lane copy
+            kernel on 1 GiB (read + write bytes), the denominator the target
+            (>= 70 %) is stated against.
+  cpu_baseline  the C/OpenMP restatement of the same ring walk (oracle/),
+            timed on this host on a smaller sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORLD = 8
+PER_RANK_BYTES = 256 << 20
+HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# the same counters' reading for a plain copy of known size; None until measured
+TRAFFIC_BYTES_PER_LAUNCH = 7.265e9
+
+# launch geometry used for the headline ("tuning")
+BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 16 << 20))
+NSLOTS = int(os.getenv("MINTCCL_BENCH_NSLOTS", 16))
+WAVES_PER_RANK = int(os.getenv("MINTCCL_BENCH_WAVES", 512))
+THREADS = int(os.getenv("MINTCCL_BENCH_THREADS", 256))
+PLACEMENT = int(os.getenv("MINTCCL_BENCH_PLACEMENT", 0))
+
+
+def cpu_baseline(seconds_budget: float = 20.0) -> dict:
+    """The oracle's C/OpenMP ring walk on a bounded sample of the workload."""
+    import numpy as np
+    from oracle import cref
+    cores = min(os.cpu_count() or 1, int(os.getenv("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    per_rank = 32 << 20                                   # 8 ranks x 32 MiB fp16
+    rng = np.random.default_rng(3000)
+    bufs = [rng.standard_normal(per_rank // 2, dtype=np.float32).astype(np.float16)
+            .view(np.uint8) for _ in range(WORLD)]
+    cref.reducescatter_wire([b.copy() for b in bufs[:WORLD]], "f16", threads=cores)   # warm-up
+    times = []
+    t_end = time.perf_counter() + seconds_budget
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 7):
+        work = [b.copy() for b in bufs]
+        t0 = time.perf_counter_ns()
+        bad = cref.reducescatter_wire(work, "f16", threads=cores)
+        times.append((time.perf_counter_ns() - t0) / 1e9)
+        assert bad == 0
+    med = sorted(times)[len(times) // 2]
+    payload = (3 * WORLD + 1) * per_rank
+    return {"value": round(payload / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"same ring walk in C/OpenMP (oracle/ll128_ref.c), 8 ranks x "
+                      f"{per_rank >> 20} MiB fp16, median of {len(times)} runs"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.getenv("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the 8 ring ranks are disjoint HBM regions "
+              "of one MI355X); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+    from mintccl_amd import primitive
+    from mintccl_amd.common import VirtualComm
+    from mintccl_amd.reducescatter import reducescatter
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # measured copy bandwidth of the library's own copy kernel, 1 GiB
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256)
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        primitive.copy128(src, dst)
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(5):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); primitive.copy128(src, dst); e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1))
+    copy_gbps = 2 * (1 << 30) / best / 1e6
+    del src, dst
+
+    # synthetic input: normal(0,1) drawn per rank (seed 3000 + rank), fp16
+    n = PER_RANK_BYTES // 2 // WORLD
+    bufs = []
+    for r in range(WORLD):
+        g = torch.Generator(device=dev).manual_seed(3000 + r)
+        bufs.append(torch.randn(WORLD, n, generator=g, device=dev, dtype=torch.float32)
+                    .to(torch.float16))
+    comm = VirtualComm(world_size=WORLD, device=dev, buff_size_=BUFF_BYTES, nslots=NSLOTS,
+                       waves_per_rank=WAVES_PER_RANK, threads_per_block=THREADS,
+                       placement=PLACEMENT)
+
+    def step():
+        comm.run(lambda r: reducescatter(bufs[r], comm))
+
+    for _ in range(args.warmup):
+        step()
+    comm.check()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()
+        step()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    comm.check()
+    kernel_ms = sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / args.steps
+
+    payload = (3 * WORLD + 1) * PER_RANK_BYTES
+    ms_per_step = wall * 1e3 / args.steps
+    value = payload / (ms_per_step / 1e3) / 1e9
+    achieved = payload / (kernel_ms / 1e3) / 1e9
+    algbw = PER_RANK_BYTES / (kernel_ms / 1e3) / 1e9
+    out = {
+        "metric": "achieved HBM GB/s and % of roofline, 8-rank LL128 reducescatter 256MiB fp16",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "ring reducescatter, LL128 (64-byte-sector tags), 8 virtual ranks "
+                               "x 256 MiB fp16 on one MI355X, in place",
+                   "world": WORLD, "per_rank_bytes": PER_RANK_BYTES, "staging_per_rank": BUFF_BYTES,
+                   "nslots": NSLOTS, "waves_per_rank": WAVES_PER_RANK, "threads": THREADS,
+                   "placement": ["spread", "local"][PLACEMENT], "grid_blocks": comm.last_grid,
+                   "payload_bytes_per_step": payload},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH},
+        "kernel_ms": round(kernel_ms, 4),
+        "copy_bw_gbps": round(copy_gbps, 1),
+        "frac_of_copy_bw": round(achieved / copy_gbps, 4),
+        "algbw_gbps": round(algbw, 1), "busbw_gbps": round(algbw * (WORLD - 1) / WORLD, 1),
+        "flag_bytes_frac_of_staging": round(8 / 128, 4),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

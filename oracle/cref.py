@@ -38,6 +38,9 @@ def lib():
         L.ref_unpack.argtypes = [vp, sz, u64, u64, ci, vp]
         L.ref_add.restype = None
         L.ref_add.argtypes = [vp, vp, vp, sz, ci]
+        L.ref_reducescatter_wire.restype = sz
+        L.ref_reducescatter_wire.argtypes = [ctypes.POINTER(vp), ci, sz, ci,
+                                             ctypes.POINTER(ci), ctypes.c_uint32, ci]
         _lib = L
     return _lib
 
@@ -68,3 +71,15 @@ def add(a, b, dtype: str) -> np.ndarray:
     item = 4 if dtype == "f32" else 2
     lib().ref_add(_p(a), _p(b), _p(out), a.size // item, DT[dtype])
     return out
+
+
+def reducescatter_wire(bufs: list, dtype: str, ring=None, epoch: int = 1, threads: int = 0) -> int:
+    """In-place ring reduce-scatter on ``bufs`` (one contiguous uint8 array of
+    ``world`` rows per rank), walked through the wire format.  Returns the
+    number of messages with wrong tags (0)."""
+    world = len(bufs)
+    ring = list(ring) if ring is not None else list(range(world)) + [0]
+    ptrs = (ctypes.c_void_p * world)(*[b.ctypes.data for b in bufs])
+    cring = (ctypes.c_int * len(ring))(*ring)
+    row = bufs[0].size // world
+    return int(lib().ref_reducescatter_wire(ptrs, world, row, DT[dtype], cring, epoch, threads))

@@ -168,3 +168,105 @@ void ref_add(const void *a, const void *b, void *out, size_t nelem, int dtype) {
         for (size_t i = 0; i < nelem; ++i) o[i] = (uint16_t)sf_add(x[i], y[i], E, M);
     }
 }
+
+/* ---- CPU baseline: ring reduce-scatter walked through the wire format -------
+ * xs[r] points at rank r's (world x row_bytes) buffer.  For every chunk c the
+ * walk of 7_reducescatter.py:54-73 is done block by block (960 raw bytes): the
+ * root's block is packed into a 1 KiB wave64 message with the step tag, the
+ * next rank checks the 16 sector tags, unpacks, adds its own block
+ * (protocol.py:142-156) and packs again; after world hops the root unpacks
+ * into its row c.  In place, like the reference.  Element addition uses the
+ * host FPU (binary32 add, one rounding back) - see oracle/ring.py for why that
+ * equals one correctly rounded addition - and OpenMP over (chunk, block).
+ * Returns the number of messages whose tags were wrong (always 0). */
+#include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static float half_to_float(uint16_t h) {
+    uint32_t s = (uint32_t)(h >> 15) << 31, e = (h >> 10) & 31, f = h & 1023, u;
+    if (e == 0) {
+        if (!f) { u = s; }
+        else { int sh = 0; while (!(f & 1024)) { f <<= 1; ++sh; }
+               u = s | ((uint32_t)(113 - sh) << 23) | ((f & 1023) << 13); }
+    } else if (e == 31) { u = s | 0x7F800000u | (f << 13); }
+    else { u = s | ((e + 112) << 23) | (f << 13); }
+    float r; memcpy(&r, &u, 4); return r;
+}
+static uint16_t float_to_half(float x) {       /* round to nearest even */
+    uint32_t u; memcpy(&u, &x, 4);
+    uint32_t s = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a >= 0x7F800000u) return (uint16_t)(s | 0x7C00u | (a > 0x7F800000u ? 0x200u : 0));
+    if (a >= 0x477FF000u) return (uint16_t)(s | 0x7C00u);           /* rounds to inf */
+    if (a < 0x38800000u) {                                           /* subnormal half */
+        if (a < 0x33000000u) return (uint16_t)s;                     /* below half of 2^-24 */
+        uint32_t e = a >> 23, m = (a & 0x7FFFFFu) | 0x800000u, sh = 126 - e;   /* 14..24 */
+        uint32_t q = m >> sh, rem = m & ((1u << sh) - 1), half = 1u << (sh - 1);
+        if (rem > half || (rem == half && (q & 1))) ++q;
+        return (uint16_t)(s | q);
+    }
+    uint32_t q = (a - 0x38000000u) >> 13, rem = a & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1))) ++q;
+    return (uint16_t)(s | q);
+}
+static uint16_t float_to_bf16(float x) {
+    uint32_t u; memcpy(&u, &x, 4);
+    if (x != x) return 0x7FC0;
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+static void add_block(const uint8_t *own, const uint8_t *recv, uint8_t *out, size_t nbytes,
+                      int dtype) {
+    if (dtype == DT_F32) {
+        for (size_t i = 0; i + 4 <= nbytes; i += 4) {
+            float a, b; memcpy(&a, own + i, 4); memcpy(&b, recv + i, 4);
+            a = a + b; memcpy(out + i, &a, 4);
+        }
+    } else if (dtype == DT_F16) {
+        for (size_t i = 0; i + 2 <= nbytes; i += 2) {
+            uint16_t a, b; memcpy(&a, own + i, 2); memcpy(&b, recv + i, 2);
+            uint16_t r = float_to_half(half_to_float(a) + half_to_float(b));
+            memcpy(out + i, &r, 2);
+        }
+    } else {
+        for (size_t i = 0; i + 2 <= nbytes; i += 2) {
+            uint16_t a, b; memcpy(&a, own + i, 2); memcpy(&b, recv + i, 2);
+            uint32_t ua = (uint32_t)a << 16, ub = (uint32_t)b << 16; float fa, fb;
+            memcpy(&fa, &ua, 4); memcpy(&fb, &ub, 4);
+            uint16_t r = float_to_bf16(fa + fb);
+            memcpy(out + i, &r, 2);
+        }
+    }
+}
+
+size_t ref_reducescatter_wire(uint8_t *const *xs, int world, size_t row_bytes, int dtype,
+                              const int *ring, uint32_t epoch, int threads) {
+    size_t nblocks = ceil_div(row_bytes, 960), bad = 0;
+#ifdef _OPENMP
+    if (threads > 0) omp_set_num_threads(threads);
+#else
+    (void)threads;
+#endif
+    long total = (long)world * (long)nblocks;
+#pragma omp parallel for schedule(static) reduction(+ : bad)
+    for (long t = 0; t < total; ++t) {
+        int c = (int)(t / (long)nblocks);
+        size_t g = (size_t)(t % (long)nblocks);
+        size_t off = g * 960, len = row_bytes - off < 960 ? row_bytes - off : 960;
+        int start = 0;
+        for (int i = 0; i < world; ++i) if (ring[i] == c) start = i;
+        uint8_t acc[960], recv[960], msg[1024];
+        uint64_t tag = ((uint64_t)epoch << 20) | (uint64_t)(g + 1);
+        memcpy(acc, xs[c] + (size_t)c * row_bytes + off, len);
+        for (int k = 1; k <= world; ++k) {
+            ref_pack(acc, len, tag, 0, LAYOUT_WAVE64, msg);
+            bad += ref_unpack(msg, len, tag, 0, LAYOUT_WAVE64, recv);
+            int r = ring[(start + k) % world];
+            if (k < world)
+                add_block(xs[r] + (size_t)c * row_bytes + off, recv, acc, len, dtype);
+            else
+                memcpy(xs[c] + (size_t)c * row_bytes + off, recv, len);
+        }
+    }
+    return bad;
+}
