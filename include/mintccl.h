@@ -62,7 +62,9 @@ typedef enum {
  * by the caller before launch).  word 0: 0 = OK, else 1 = a bounded wait ran
  * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
  * that gave up; word 2: step it waited for; word 3: abort flag polled by all
- * other waits.  The reference has no abort path (common.py:106 is unused). */
+ * other waits.  Error code 2: a block did not run on XCD (block index % 8), which
+ * cache_policy 2 relies on; word 2 then holds the XCD it ran on.
+ * The reference has no abort path (common.py:106 is unused). */
 #define MINT_STATUS_WORDS 4
 
 /* One ring collective over `world` virtual ranks of one GPU.  It stands for the
@@ -90,7 +92,9 @@ typedef struct {
     uint32_t waves_per_channel_group; /* wave-channels per (pipeline, hop) */
     uint32_t threads_per_block;       /* multiple of 64 */
     int32_t placement;     /* mint_placement */
-    int32_t cache_policy;  /* 0 agent scope (sc1), 1 system scope (sc0 sc1) */
+    int32_t cache_policy;  /* how staging is accessed: 0 agent scope (sc1),
+                              1 system scope (sc0 sc1), 2 XCD-local (stores
+                              stay in the XCD's L2; needs MINT_PLACE_LOCAL) */
     uint32_t flag_epoch;   /* 1..4095; must differ from every earlier launch
                               that used the same staging memory since that
                               memory was last zeroed */
@@ -98,6 +102,12 @@ typedef struct {
     uint64_t status;       /* device address of MINT_STATUS_WORDS uint64 */
     uint32_t debug_skip_origin; /* testing: origin hop sends nothing */
     uint32_t reserved;
+    uint64_t debug_stats;  /* 0.  A library built with -DMINT_RING_STATS takes
+                              the device address of (hops + 1) x 8 zeroed
+                              uint64 and fills, per position, {groups,
+                              re-polls, ticks waiting for credit, ticks
+                              polling, ticks total, wavefronts, 0, 0}; a tick
+                              is 10 ns.  Other builds reject non-zero. */
 } mint_ring_op;
 
 int mint_version(void);
@@ -153,7 +163,8 @@ int mint_ring_launch(const mint_ring_op* op, void* stream);
  * line is tested (one flag per 128-byte line, the reference's assumption,
  * protocol.py:31-35).  counters: device uint64[8] = {lines checked, torn
  * lines, polls, timeouts, torn lines whose first sector alone was stale, 0..}.
- * flag_epoch is 1..4095. */
+ * flag_epoch is 1..4095.  With MINT_PLACE_LOCAL the pair count must be a
+ * multiple of 32 (whole blocks per XCD). */
 int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,
                          int cache_policy, int placement, int per_sector, uint32_t flag_epoch,
                          uint32_t spin_budget, void* counters, void* stream);

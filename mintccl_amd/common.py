@@ -53,6 +53,10 @@ def protocol_env() -> int:
         os.getenv("MINTCCL_PROTOCOL", "ll128").lower()]
 
 
+def cache_policy_env() -> int:
+    return {"agent": 0, "system": 1, "xcd": 2}[os.getenv("MINTCCL_CACHE", "agent").lower()]
+
+
 def placement_env() -> int:
     return {"spread": _lib.PLACE_SPREAD, "local": _lib.PLACE_LOCAL}[
         os.getenv("MINTCCL_PLACEMENT", "spread").lower()]
@@ -100,7 +104,12 @@ class Timer:
 
 
 class RingTimeout(RuntimeError):
-    """A bounded wait inside the ring kernel ran out (status word 0 != 0)."""
+    """A bounded wait inside the ring kernel ran out (status word 0 == 1)."""
+
+
+class PlacementError(RuntimeError):
+    """cache_policy 2 was used but a block did not run on the XCD the
+    round-robin dealing predicts (status word 0 == 2)."""
 
 
 def _largest_divisor_at_most(n: int, cap: int) -> int:
@@ -125,7 +134,7 @@ class VirtualComm:
                  buff_size_: int | None = None, nslots: int | None = None,
                  protocol: int | None = None, placement: int | None = None,
                  waves_per_rank: int | None = None, threads_per_block: int | None = None,
-                 cache_policy: int = 0, spin_budget: int = 0) -> None:
+                 cache_policy: int | None = None, spin_budget: int = 0) -> None:
         self.world_size = world_size if world_size is not None else world_size_env()
         if not 1 <= self.world_size <= _lib.MAX_RANKS:
             raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
@@ -142,7 +151,9 @@ class VirtualComm:
                                else max(1, num_blocks() * num_warps() // 2))
         self.threads_per_block = (threads_per_block if threads_per_block is not None
                                   else _env_int("MINTCCL_THREADS", 256))
-        self.cache_policy = cache_policy
+        self.cache_policy = cache_policy if cache_policy is not None else cache_policy_env()
+        if self.cache_policy == 2 and self.placement != _lib.PLACE_LOCAL:
+            raise ValueError("the XCD-local cache policy needs the local placement")
         self.spin_budget = spin_budget
         self._lib = _lib.lib()          # fails loudly if the extension is missing
         # slots + credit words (never more than slot_bytes / 4), zeroed: flag 0
@@ -152,6 +163,7 @@ class VirtualComm:
         self.staging = torch.zeros(self.world_size * self.rank_stride, dtype=torch.uint8,
                                    device=self.device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int64, device=self.device)
+        self.stats = None              # set to a zeroed int64[(hops + 1) * 8] tensor to collect wait accounting
         self.epoch = 0
         self._tls = threading.local()
         self._pending: dict = {}
@@ -236,6 +248,7 @@ class VirtualComm:
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
         d.debug_skip_origin = int(skip_origin)
+        d.debug_stats = self.stats.data_ptr() if self.stats is not None else NULL
         return d
 
     def launch(self, d: _lib.RingOp) -> None:
@@ -259,6 +272,11 @@ class VirtualComm:
         if st[0] != 0:
             self.status.zero_()
             who = st[1]
+            if st[0] == 2:
+                raise PlacementError(
+                    f"block of pipeline {who >> 32}, position {(who >> 16) & 0xFFFF} ran on XCD "
+                    f"{st[2]}: thread blocks are not dealt round-robin over the XCDs here; "
+                    "use cache_policy 0")
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
                 f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]}")

@@ -150,7 +150,7 @@ __device__ __forceinline__ uint32_t probe_word(uint32_t tag, uint32_t lane, uint
 }
 constexpr uint32_t kProbeDepth = 4;   // blocks per pair, reused round-robin
 
-template <int CP>
+template <int LDCP, int STCP>
 __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint32_t pairs,
                                                          uint32_t iters, int placement,
                                                          int per_sector, uint32_t epoch,
@@ -160,8 +160,15 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
     const uint32_t wpb = blockDim.x >> 6;
     const uint32_t pair_blocks = (pairs + wpb - 1) / wpb;
     uint32_t pb; bool producer;
-    if (placement == 1) { pb = blockIdx.x % pair_blocks; producer = blockIdx.x < pair_blocks; }
-    else                { pb = blockIdx.x >> 1;          producer = !(blockIdx.x & 1u); }
+    if (placement == 1) {
+        // producer and consumer of a pair are consecutive blocks of the same XCD
+        const uint32_t xcd = blockIdx.x % 8u, y = blockIdx.x / 8u;
+        pb = (y >> 1) * 8u + xcd;
+        producer = !(y & 1u);
+    } else {
+        pb = blockIdx.x >> 1;
+        producer = !(blockIdx.x & 1u);
+    }
     const uint32_t pair = pb * wpb + (uint32_t)wave_in_block();
     if (pair >= pairs) return;
     const uint32_t data_bytes = pairs * kProbeDepth * kBlockMsg;
@@ -186,13 +193,13 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
             }
             u32x4 v = {probe_word(tag, m.lane, 0), probe_word(tag, m.lane, 1),
                        probe_word(tag, m.lane, 2), probe_word(tag, m.lane, 3)};
-            ll_send<CP>(win, off, v, tag, m);
+            ll_send<STCP>(win, off, v, tag, m);
         } else {
             u32x4 v; bool ok = false;
             for (uint32_t spins = 0; spins <= budget; ++spins) {
                 compiler_fence();
                 ++polls;
-                v = ld128<CP>(win, off + m.lane * 16u);
+                v = ld128<LDCP>(win, off + m.lane * 16u);
                 const bool tested = m.flag_lane && (per_sector || (m.sector & 1u));
                 if (wave_all(!tested || v.w == tag)) { ok = true; break; }
                 __builtin_amdgcn_s_sleep(1);
@@ -208,7 +215,10 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
                 first_half += line == 0x0Fu ? 1u : 0u;   // exactly the first sector stale
             }
             checked += 8u;
-            if (lane_id() == 0) st64_agent(tail, flag_hi | (uint64_t)(t + 1));
+            if (lane_id() == 0) {
+                if (STCP == CP_NONE) st64_local(tail, flag_hi | (uint64_t)(t + 1));
+                else st64_agent(tail, flag_hi | (uint64_t)(t + 1));
+            }
         }
     }
     if (lane_id() == 0) {

@@ -45,7 +45,9 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
     if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
-    if (op->cache_policy != 0 && op->cache_policy != 1) return MINT_ERR_ARG;
+    if (op->cache_policy < 0 || op->cache_policy > 2) return MINT_ERR_ARG;
+    // XCD-local staging only makes sense when every hop of a channel shares an XCD
+    if (op->cache_policy == 2 && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
     if (op->placement != MINT_PLACE_SPREAD && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
     if (op->flag_epoch == 0 || op->flag_epoch > kMaxEpoch || !op->status) return MINT_ERR_ARG;
     if (op->threads_per_block == 0 || op->threads_per_block % 64 || op->threads_per_block > 512)
@@ -148,6 +150,12 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
     a.status = reinterpret_cast<uint64_t*>(op->status);
     a.skip_origin = op->debug_skip_origin;
+#ifdef MINT_RING_STATS
+    a.stats = reinterpret_cast<uint64_t*>(op->debug_stats);
+#else
+    if (op->debug_stats) return MINT_ERR_ARG;   // this build does not collect wait accounting
+    a.stats = nullptr;
+#endif
     a.placement = op->placement;
 
     const int waves_per_block = (int)op->threads_per_block / 64;
@@ -155,6 +163,9 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     if (a.waves < waves_per_block) plan->threads = a.waves * 64;
     a.blocks_per_group = (a.waves * 64 + plan->threads - 1) / plan->threads;
     plan->blocks = a.pipes * (a.hops + 1) * a.blocks_per_group;
+    // the XCD-local mapping deals whole channels to XCDs
+    if (op->placement == MINT_PLACE_LOCAL && (a.pipes * a.blocks_per_group) % kXcds)
+        return MINT_ERR_GEOMETRY;
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
     return MINT_OK;
 }
@@ -179,8 +190,11 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
 }
 template <int PROTO, int DT>
 int launch_ring_cp(const Plan& plan, int cache_policy, hipStream_t stream) {
-    return cache_policy == 0 ? launch_ring_u<PROTO, DT, CP_AGENT>(plan, stream)
-                             : launch_ring_u<PROTO, DT, CP_SYSTEM>(plan, stream);
+    switch (cache_policy) {
+        case 0: return launch_ring_u<PROTO, DT, 0>(plan, stream);
+        case 1: return launch_ring_u<PROTO, DT, 1>(plan, stream);
+        default: return launch_ring_u<PROTO, DT, 2>(plan, stream);
+    }
 }
 template <int PROTO>
 int launch_ring_dt(const Plan& plan, int dtype, int cache_policy, hipStream_t stream) {
@@ -376,11 +390,15 @@ int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int ite
         flag_epoch == 0 || flag_epoch > kMaxEpoch)
         return MINT_ERR_ARG;
     if (!aligned16(staging)) return MINT_ERR_ALIGN;
-    if (cache_policy != 0 && cache_policy != 1) return MINT_ERR_ARG;
+    if (cache_policy < 0 || cache_policy > 2) return MINT_ERR_ARG;
+    if (cache_policy == 2 && placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
     const size_t need = (size_t)pairs * (kProbeDepth * kBlockMsg + 128u);
     if (staging_bytes < need || need >= (1ull << 31)) return MINT_ERR_ARG;
     const int wpb = 4, pair_blocks = (pairs + wpb - 1) / wpb, blocks = 2 * pair_blocks;
-    auto kernel = cache_policy == 0 ? torn_probe_kernel<CP_AGENT> : torn_probe_kernel<CP_SYSTEM>;
+    if (placement == MINT_PLACE_LOCAL && pair_blocks % kXcds) return MINT_ERR_GEOMETRY;
+    auto kernel = cache_policy == 0   ? torn_probe_kernel<Policy<0>::LD, Policy<0>::ST>
+                  : cache_policy == 1 ? torn_probe_kernel<Policy<1>::LD, Policy<1>::ST>
+                                      : torn_probe_kernel<Policy<2>::LD, Policy<2>::ST>;
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess)
         return MINT_ERR_HIP;

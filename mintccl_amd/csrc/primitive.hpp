@@ -81,6 +81,12 @@ __device__ __forceinline__ uint64_t ld64_agent(const uint64_t* p) {
 __device__ __forceinline__ void st64_agent(uint64_t* p, uint64_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Plain 64-bit store (no scope bits): stays in the L2 of the XCD that runs the
+// wave.  Relaxed atomic at wavefront scope, so the compiler keeps it whole and
+// in program order with respect to other atomics.
+__device__ __forceinline__ void st64_local(uint64_t* p, uint64_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+}
 __device__ __forceinline__ uint64_t ld64_acquire(const uint64_t* p) {
     return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
 }

@@ -112,6 +112,37 @@ __device__ __forceinline__ u32x4 ll_load_raw(const uint8_t* row, uint64_t row_by
     }
     return v;
 }
+// The same through a buffer window, with an explicit cache policy (rows of
+// less than 4 GiB; the ragged last block still goes through the pointer).
+template <int CP>
+__device__ __forceinline__ u32x4 ll_load_raw_w(const Window& win, const uint8_t* row,
+                                               uint64_t row_bytes, uint32_t g, const LaneMap& m) {
+    const uint64_t base = (uint64_t)g * kBlockRawLL;
+    u32x4 v;
+    if (base + kBlockRawLL <= row_bytes) {
+        const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
+        v = ld128<CP>(win, (uint32_t)base + off);
+        if (m.flag_lane) { v.x = v.y; v.y = v.z; v.z = v.w; }
+    } else {
+        v = load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
+    }
+    return v;
+}
+template <int CP>
+__device__ __forceinline__ void ll_save_raw_w(const Window& win, uint8_t* row, uint64_t row_bytes,
+                                              uint32_t g, const LaneMap& m, u32x4 v) {
+    const uint64_t base = (uint64_t)g * kBlockRawLL;
+    if (base + kBlockRawLL <= row_bytes) {
+        if (!m.flag_lane) {
+            st128<CP>(win, (uint32_t)base + m.raw_off, v);
+        } else {
+            u32x3 h = {v.x, v.y, v.z};
+            __builtin_amdgcn_raw_buffer_store_b96(h, win.rsrc, (int)((uint32_t)base + m.raw_off), 0, CP);
+        }
+    } else {
+        store_guarded(row, base + m.raw_off, m.raw_len, row_bytes, v);
+    }
+}
 // save_ll128 (protocol.py:87-100): registers -> raw block g of a row.
 __device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, uint32_t g,
                                             const LaneMap& m, u32x4 v) {

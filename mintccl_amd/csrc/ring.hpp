@@ -41,6 +41,7 @@ enum : int { PROTO_LL128 = 0, PROTO_SIMPLE = 1 };
 enum : int { PLACE_SPREAD = 0, PLACE_LOCAL = 1 };
 
 constexpr int kMaxRanks = 8;
+constexpr int kXcds = 8;                  // XCDs of an MI355X; blocks are dealt over them round-robin
 constexpr uint32_t kCreditStride = 256;   // per wave-channel: line 0 tail, line 1 head
 
 struct RingArgs {
@@ -63,6 +64,7 @@ struct RingArgs {
     uint32_t epoch, spin_budget;
     uint64_t* status;
     uint32_t skip_origin;
+    uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
 };
 
 struct Role {
@@ -86,17 +88,22 @@ __device__ __forceinline__ Role role_of(const RingArgs& a, int p, int h) {
     return r;
 }
 
-// First waiter that gives up records who it was; everybody else sees word 3.
-__device__ __forceinline__ void report_timeout(uint64_t* status, int p, int h, int w,
-                                               uint64_t step) {
+// First wavefront that gives up records why (1 = a bounded wait ran out,
+// 2 = block not on the expected XCD) and who it was; everybody else sees word 3.
+__device__ __forceinline__ void report_error(uint64_t* status, uint64_t code, int p, int h, int w,
+                                             uint64_t detail) {
     if (lane_id() == 0) {
         unsigned long long* s = reinterpret_cast<unsigned long long*>(status);
-        if (atomicCAS(s, 0ull, 1ull) == 0ull) {
+        if (atomicCAS(s, 0ull, (unsigned long long)code) == 0ull) {
             st64_agent(status + 1, ((uint64_t)p << 32) | ((uint64_t)h << 16) | (uint64_t)w);
-            st64_agent(status + 2, step);
+            st64_agent(status + 2, detail);
         }
         st64_agent(status + 3, 1ull);
     }
+}
+__device__ __forceinline__ void report_timeout(uint64_t* status, int p, int h, int w,
+                                               uint64_t step) {
+    report_error(status, 1, p, h, w, step);
 }
 __device__ __forceinline__ bool aborted(const uint64_t* status) {
     return __builtin_amdgcn_readfirstlane((uint32_t)ld64_agent(status + 3)) != 0u;
@@ -120,17 +127,52 @@ __device__ __forceinline__ bool wait_count(const uint64_t* word, uint32_t epoch,
     }
 }
 
-template <int PROTO, int DT, int CP, int U>
+// How staging memory is accessed.  The sector tags make any choice safe: a
+// stale or partially visible sector fails its tag test and is polled again,
+// so a wrong policy costs time (or a reported time-out), never data.
+//   0  agent scope: loads and stores miss / write through the per-XCD L2, so
+//      producer and consumer may sit on different XCDs
+//   1  system scope
+//   2  XCD-local: stores (and credit words) carry no scope bits and stay in
+//      the L2 of the XCD; loads are agent scope, which skips the per-CU L1 and
+//      is served by that L2 while the line is still there.  Only valid with
+//      PLACE_LOCAL, where all hops of a channel share one XCD; the kernel
+//      checks that blocks really are dealt round-robin over the XCDs.
+//      (Measured alternatives: nt loads behave like sc1 loads; plain and sc0
+//      loads keep hitting stale L1 lines and time out, with or without
+//      buffer_inv sc0.)
+template <int CPI> struct Policy;
+template <> struct Policy<0> { static constexpr int LD = CP_SC1, ST = CP_SC1; };
+template <> struct Policy<1> { static constexpr int LD = CP_SYSTEM, ST = CP_SYSTEM; };
+template <> struct Policy<2> { static constexpr int LD = CP_SC1, ST = CP_NONE; };
+
+template <int PROTO, int DT, int CPI, int U>
 __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
+    constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
     const int npos = a.hops + 1;
-    const int channels = a.pipes * a.blocks_per_group;
     const int x = (int)blockIdx.x;
     int c, h;
-    if (a.placement == PLACE_LOCAL) { c = x % channels; h = x / channels; }
-    else                            { h = x % npos;     c = x / npos; }
+    if (a.placement == PLACE_LOCAL) {
+        // blocks are dealt round-robin over the XCDs: block x runs on XCD
+        // x % 8.  Give XCD d the channels c with c % 8 == d and let the blocks
+        // it receives walk through the positions of one channel after the
+        // other, so a channel's whole ring shares one L2, is dispatched
+        // together, and every CU hosts a mix of positions.
+        const int xcd = x % kXcds, y = x / kXcds;
+        h = y % npos;
+        c = (y / npos) * kXcds + xcd;
+    } else {
+        h = x % npos;
+        c = x / npos;
+    }
     const int p = c / a.blocks_per_group;
     const int w = (c % a.blocks_per_group) * (int)(blockDim.x >> 6) + wave_in_block();
     if (w >= a.waves) return;
+    if (CPI == 2 && xcc_id() != x % kXcds) {
+        // the XCD-local policy rests on block x running on XCD x % 8
+        report_error(a.status, 2, p, h, w, (uint64_t)xcc_id());
+        return;
+    }
     const Role role = role_of(a, p, h);
     if (h == 0 && a.skip_origin) return;
 
@@ -138,6 +180,9 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const uint64_t row_off = (uint64_t)p * a.row_stride;
     const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
     uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
+#if defined(MINT_RAW_LD_CP) || defined(MINT_RAW_ST_CP)
+    const Window in_w(in_row, (uint32_t)a.row_bytes), out_w(out_row, (uint32_t)a.row_bytes);
+#endif
     const uint32_t ring_bytes = a.nslots * a.slot_bytes;
     const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
     const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);
@@ -149,119 +194,182 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
 
     const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
     const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
+    const uint32_t groups_per_step = K / U;
+    const uint32_t ngroups = a.steps * groups_per_step;
     uint32_t credits_seen = 0, head_seen = 0;
+    // wait accounting, 10 ns ticks: only in a library built with
+    // -DMINT_RING_STATS (it costs scalar registers, hence occupancy)
+#ifdef MINT_RING_STATS
+    const bool timing = a.stats != nullptr;
+#else
+    constexpr bool timing = false;
+#endif
+    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
+    const uint64_t t_begin = timing ? wall_clock64() : 0;
 
-    for (uint32_t s = 0; s < a.steps; ++s) {
-        const uint32_t slot_off = (s % a.nslots) * a.slot_bytes + (uint32_t)p * a.step_msg;
-        const uint32_t g0 = s * a.step_blocks;
-        const uint32_t tag = (a.epoch << 20) | (s + 1u);
-        if (role.send && s >= a.nslots) {
-            if (!wait_count(nxt_tail, a.epoch, s - a.nslots + 1, credits_seen, a.spin_budget,
-                            a.status, false)) {
-                report_timeout(a.status, p, h, w, s);
-                return;
+    // Block indices of group n: U blocks of this wave-channel inside step n / groups_per_step.
+    struct Group { uint32_t step, idx[U], g[U]; bool valid[U], first, last; };
+    auto group_of = [&](uint32_t n) {
+        Group q;
+        q.step = n / groups_per_step;
+        const uint32_t k0 = (n % groups_per_step) * (uint32_t)U;
+        q.first = k0 == 0;
+        q.last = k0 + (uint32_t)U >= K;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            q.idx[u] = (k0 + (uint32_t)u) * W + (uint32_t)w;
+            q.g[u] = q.step * a.step_blocks + q.idx[u];
+            q.valid[u] = q.g[u] < a.nblocks;
+        }
+        return q;
+    };
+    // load_ll128 of the wave's own rows for one group.
+    auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v[u] = u32x4{0u, 0u, 0u, 0u};
+            if (!q.valid[u]) continue;
+            if (PROTO == PROTO_LL128) {
+#ifdef MINT_RAW_LD_CP
+                v[u] = ll_load_raw_w<MINT_RAW_LD_CP>(in_w, in_row, a.row_bytes, q.g[u], m);
+#else
+                v[u] = ll_load_raw(in_row, a.row_bytes, q.g[u], m);
+#endif
+            } else {
+                const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
+                v[u] = off + 16u <= a.row_bytes ? ld128_stream(in_row + off)
+                                               : load_guarded(in_row, off, 16u, a.row_bytes);
             }
         }
-        if (PROTO == PROTO_SIMPLE && role.recv) {
+    };
+
+    // The own rows do not depend on anybody, so they are fetched one group
+    // ahead: the load for group n + 1 is issued right after the first poll of
+    // group n (younger than the poll, so waiting for the poll does not wait
+    // for it) and has a whole group's time to come back from HBM.
+    u32x4 v[U], vnext[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
+    if (role.load && ngroups) load_own(group_of(0), v);
+
+    for (uint32_t n = 0; n < ngroups; ++n) {
+        const Group q = group_of(n);
+        const uint32_t s = q.step;
+        const uint32_t slot_off = (s % a.nslots) * a.slot_bytes + (uint32_t)p * a.step_msg;
+        const uint32_t tag = (a.epoch << 20) | (s + 1u);
+        // wait_ll128 (protocol.py:161-180): the credit for the slot this step
+        // goes into is only needed before the send, so its load is issued
+        // here, ahead of the polls, and looked at after them.
+        const uint32_t need = s >= a.nslots ? s - a.nslots + 1 : 0;
+        const bool ask_credit = q.first && role.send && credits_seen < need;
+        uint64_t credit_word = 0;
+        if (ask_credit) credit_word = ld64_agent(nxt_tail);
+        if (q.first && PROTO == PROTO_SIMPLE && role.recv) {
+            const uint64_t t0 = timing ? wall_clock64() : 0;
             if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status, true)) {
                 report_timeout(a.status, p, h, w, s);
                 return;
             }
+            if (timing) t_credit += wall_clock64() - t0;
         }
-        for (uint32_t k0 = 0; k0 < K; k0 += U) {
-            uint32_t idx[U], g[U];
-            bool valid[U];
-            u32x4 v[U];
+        u32x4 r[U];
+        const uint64_t t1 = timing ? wall_clock64() : 0;
+        if (role.recv) {
+            // first poll of recv_ll128 (protocol.py:102-130): loads only
+            compiler_fence();
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                idx[u] = (k0 + (uint32_t)u) * W + (uint32_t)w;
-                g[u] = g0 + idx[u];
-                valid[u] = g[u] < a.nblocks;
-                v[u] = u32x4{0u, 0u, 0u, 0u};
-            }
-            if (!valid[0]) break;
-            if (role.load) {
+            for (int u = 0; u < U; ++u)
+                if (q.valid[u])
+                    r[u] = ld128<LDCP>(own, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u);
+        }
+        if (role.load && n + 1 < ngroups) load_own(group_of(n + 1), vnext);
+        if (role.recv && PROTO == PROTO_LL128) {
+            uint32_t pending = 0;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (q.valid[u] && !wave_all(!m.flag_lane || r[u].w == tag)) pending |= 1u << u;
+            for (uint32_t spins = 0; pending; ++spins) {
+                if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
+                    report_timeout(a.status, p, h, w, s);
+                    return;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                compiler_fence();
+                ++n_repoll;
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    if (!valid[u]) continue;
-                    if (PROTO == PROTO_LL128) {
-                        v[u] = ll_load_raw(in_row, a.row_bytes, g[u], m);
-                    } else {
-                        const uint64_t off = (uint64_t)g[u] * kBlockRawSimple + m.lane * 16u;
-                        v[u] = off + 16u <= a.row_bytes ? ld128_stream(in_row + off)
-                                                       : load_guarded(in_row, off, 16u, a.row_bytes);
-                    }
+                    if (!(pending & (1u << u))) continue;
+                    if (ll_poll<LDCP>(own, slot_off + q.idx[u] * kBlockMsg, tag, m, r[u]))
+                        pending &= ~(1u << u);
                 }
             }
+        }
+        if (timing) { t_poll += wall_clock64() - t1; ++n_groups; }
+        if (ask_credit) {
+            const uint64_t t0 = timing ? wall_clock64() : 0;
+            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(credit_word >> 32));
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)credit_word);
+            if (hi == a.epoch && lo >= need) {
+                credits_seen = lo;
+            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget, a.status,
+                                   false)) {
+                report_timeout(a.status, p, h, w, s);
+                return;
+            }
+            if (timing) t_credit += wall_clock64() - t0;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!q.valid[u]) continue;
             if (role.recv) {
-                u32x4 r[U];
-                if (PROTO == PROTO_LL128) {
-                    uint32_t pending = 0;
-#pragma unroll
-                    for (int u = 0; u < U; ++u) pending |= valid[u] ? 1u << u : 0u;
-                    for (uint32_t spins = 0; pending; ++spins) {
-                        compiler_fence();
-#pragma unroll
-                        for (int u = 0; u < U; ++u) {
-                            if (!(pending & (1u << u))) continue;
-                            if (ll_poll<CP>(own, slot_off + idx[u] * kBlockMsg, tag, m, r[u]))
-                                pending &= ~(1u << u);
-                        }
-                        if (!pending) break;
-                        if (spins >= a.spin_budget ||
-                            ((spins & 63u) == 63u && aborted(a.status))) {
-                            report_timeout(a.status, p, h, w, s);
-                            return;
-                        }
-                        __builtin_amdgcn_s_sleep(1);
-                    }
+                if constexpr (DT != DT_BYTES) {
+                    v[u] = role.reduce ? ll_comp<DT>(v[u], r[u]) : r[u];
                 } else {
-#pragma unroll
-                    for (int u = 0; u < U; ++u)
-                        if (valid[u])
-                            r[u] = ld128<CP>(own, slot_off + idx[u] * kBlockMsg + m.lane * 16u);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (!valid[u]) continue;
-                    if constexpr (DT != DT_BYTES) {
-                        v[u] = role.reduce ? ll_comp<DT>(v[u], r[u]) : r[u];
-                    } else {
-                        v[u] = r[u];
-                    }
+                    v[u] = r[u];
                 }
             }
             if (role.save) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (!valid[u]) continue;
-                    if (PROTO == PROTO_LL128) {
-                        ll_save_raw(out_row, a.row_bytes, g[u], m, v[u]);
-                    } else {
-                        const uint64_t off = (uint64_t)g[u] * kBlockRawSimple + m.lane * 16u;
-                        if (off + 16u <= a.row_bytes) st128_stream(out_row + off, v[u]);
-                        else store_guarded(out_row, off, 16u, a.row_bytes, v[u]);
-                    }
+                if (PROTO == PROTO_LL128) {
+#ifdef MINT_RAW_ST_CP
+                    ll_save_raw_w<MINT_RAW_ST_CP>(out_w, out_row, a.row_bytes, q.g[u], m, v[u]);
+#else
+                    ll_save_raw(out_row, a.row_bytes, q.g[u], m, v[u]);
+#endif
+                } else {
+                    const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
+                    if (off + 16u <= a.row_bytes) st128_stream(out_row + off, v[u]);
+                    else store_guarded(out_row, off, 16u, a.row_bytes, v[u]);
                 }
             }
             if (role.send) {
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (!valid[u]) continue;
-                    if (PROTO == PROTO_LL128) {
-                        ll_send<CP>(nxt, slot_off + idx[u] * kBlockMsg, v[u], tag, m);
-                    } else {
-                        st128<CP>(nxt, slot_off + idx[u] * kBlockMsg + m.lane * 16u, v[u]);
-                    }
-                }
+                if (PROTO == PROTO_LL128)
+                    ll_send<STCP>(nxt, slot_off + q.idx[u] * kBlockMsg, v[u], tag, m);
+                else
+                    st128<STCP>(nxt, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
             }
         }
-        // post_ll128 (protocol.py:183-189): this wave-channel has taken every
-        // line of step s out of its slot (the loads have returned: their
-        // values were tested / used above).
-        if (role.recv && lane_id() == 0) st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
-        if (PROTO == PROTO_SIMPLE && role.send && lane_id() == 0)
-            st64_release(nxt_head, flag_hi | (uint64_t)(s + 1));
+        if (q.last) {
+            // post_ll128 (protocol.py:183-189): this wave-channel has taken every
+            // line of step s out of its slot (the loads have returned: their
+            // values were tested / used above).
+            if (role.recv && lane_id() == 0) {
+                if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
+                else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
+            }
+            if (PROTO == PROTO_SIMPLE && role.send && lane_id() == 0)
+                st64_release(nxt_head, flag_hi | (uint64_t)(s + 1));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = vnext[u];
+    }
+    if (timing && lane_id() == 0) {
+        unsigned long long* st = reinterpret_cast<unsigned long long*>(a.stats) + 8 * h;
+        atomicAdd(st + 0, (unsigned long long)n_groups);
+        atomicAdd(st + 1, (unsigned long long)n_repoll);
+        atomicAdd(st + 2, (unsigned long long)t_credit);
+        atomicAdd(st + 3, (unsigned long long)t_poll);
+        atomicAdd(st + 4, (unsigned long long)(wall_clock64() - t_begin));
+        atomicAdd(st + 5, 1ull);
     }
 }
 

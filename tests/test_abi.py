@@ -102,7 +102,12 @@ def test_plan_geometry_without_a_gpu():
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
     (dict(op=7), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
     (dict(dtype=_lib.BYTES), _lib.ERR_ARG),          # a reduction needs a real dtype
-    (dict(flag_epoch=0), _lib.ERR_ARG), (dict(status=0), _lib.ERR_ARG),
+    (dict(flag_epoch=0), _lib.ERR_ARG), (dict(flag_epoch=4096), _lib.ERR_ARG),
+    (dict(status=0), _lib.ERR_ARG), (dict(cache_policy=3), _lib.ERR_ARG),
+    (dict(cache_policy=2, placement=0), _lib.ERR_ARG),   # XCD-local staging needs the local placement
+    (dict(debug_stats=0x1000), _lib.ERR_ARG),            # this build collects no wait accounting
+    (dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, waves_per_channel_group=16),
+     _lib.ERR_GEOMETRY),                                 # 4 channels cannot be dealt to 8 XCDs
     (dict(threads_per_block=100), _lib.ERR_ARG),
     (dict(slot_bytes=(512 << 10) + 512), _lib.ERR_GEOMETRY),
     (dict(slot_bytes=4096), _lib.ERR_GEOMETRY),        # less than one block per pipeline

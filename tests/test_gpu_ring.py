@@ -63,12 +63,12 @@ def test_reducescatter_f16(dev, world, n):
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("proto", [0, 1])
-@pytest.mark.parametrize("place", [0, 1])
-def test_reducescatter_dtypes_protocols_placements(dev, dt, proto, place):
+@pytest.mark.parametrize("place,cp", [(0, 0), (1, 0), (0, 1), (1, 2)])
+def test_reducescatter_dtypes_protocols_placements(dev, dt, proto, place, cp):
     world, n = 8, 65536 + 8
     host = rank_rows(world, n, dt)
     bufs = [h.to(dev) for h in host]
-    comm = make_comm(world, protocol=proto, placement=place)
+    comm = make_comm(world, protocol=proto, placement=place, cache_policy=cp)
     run_reducescatter(comm, bufs)
     assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], dt))
 
@@ -145,6 +145,36 @@ def test_allgather(dev, world, n, proto):
     comm = make_comm(world, protocol=proto)
     run_allgather(comm, bufs)
     assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+
+
+@pytest.mark.parametrize("world", [2, 4, 8])
+def test_xcd_local_policy_all_collectives(dev, world):
+    # stores that stay in one XCD's L2: every collective, ragged sizes, many
+    # steps through 2 small slots
+    comm = make_comm(world, placement=1, cache_policy=2, buff_size_=2 * 64 * 1024, nslots=2,
+                     waves_per_rank=64)
+    n = 200008
+    host = rank_rows(world, n, "f16")
+    bufs = [h.to(dev) for h in host]
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+    host = [uniform(world * n, -1.0, 1.0, 4 + r).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    run_allgather(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    host = [normal(300001, 3000 + r) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    run_reduce(comm, bufs, world - 1)
+    assert same(bufs, ring.reduce([as_bytes(h) for h in host], world - 1, "f16"))
+    bufs = [h.to(dev) for h in host]
+    run_broadcast(comm, bufs, 0)
+    for b in bufs:
+        assert torch.equal(b.cpu(), host[0])
+
+
+def test_xcd_local_policy_needs_local_placement(dev):
+    with pytest.raises(ValueError):
+        make_comm(8, placement=0, cache_policy=2)
 
 
 def test_permuted_ring(dev):
@@ -227,8 +257,7 @@ def run_probe(lib, dev, pairs, iters, cp, place, per_sector):
     return cnt.cpu().tolist()
 
 
-@pytest.mark.parametrize("cp", [0, 1])
-@pytest.mark.parametrize("place", [0, 1])
+@pytest.mark.parametrize("cp,place", [(0, 0), (0, 1), (1, 0), (1, 1), (2, 1)])
 def test_no_torn_sectors(lib, dev, cp, place):
     # every 64-byte sector carries its tag and a payload that is a function of
     # the tag: once all 16 tags of a block are seen, every byte must belong
