@@ -14,7 +14,7 @@ are already resident in HBM.  Prints ONE JSON line:
   roofline  the same bytes over the kernel's own duration (HIP events on the
             launch stream), against the 8 TB/s HBM peak.  `traffic` is the HBM
             bytes per launch measured with rocprofv3 counters
-            (profiles/reducescatter_ll128_f16_256mib_pmc.txt).
+            (profiles/reducescatter_ll128_f16_256mib_*_pmc.txt).
   copy_*    measured HBM copy bandwidth of the library's own 16 B / lane copy
             kernel on 1 GiB (read + write bytes), the denominator the target
             (>= 70 %) is stated against.
@@ -37,14 +37,17 @@ PER_RANK_BYTES = 256 << 20
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
 # the same counters' reading for a plain copy of known size; None until measured
-TRAFFIC_BYTES_PER_LAUNCH = 7.265e9
+TRAFFIC_BYTES_PER_LAUNCH = {2: 2.931e9, 0: 7.780e9}
 
-# launch geometry used for the headline ("tuning")
-BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 16 << 20))
-NSLOTS = int(os.getenv("MINTCCL_BENCH_NSLOTS", 16))
+# launch geometry used for the headline: 3 slots of
+# 512 KiB per rank so that all staging of an XCD's channels stays in its 4 MiB
+# L2, 64 wave-channels per (chunk, hop), every hop of a channel on one XCD
+BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 3 * 512 * 1024))
+NSLOTS = int(os.getenv("MINTCCL_BENCH_NSLOTS", 3))
 WAVES_PER_RANK = int(os.getenv("MINTCCL_BENCH_WAVES", 512))
 THREADS = int(os.getenv("MINTCCL_BENCH_THREADS", 256))
-PLACEMENT = int(os.getenv("MINTCCL_BENCH_PLACEMENT", 0))
+PLACEMENT = int(os.getenv("MINTCCL_BENCH_PLACEMENT", 1))      # 0 spread, 1 local
+CACHE_POLICY = int(os.getenv("MINTCCL_BENCH_CACHE", 2))       # 0 agent, 1 system, 2 XCD-local
 
 
 def cpu_baseline(seconds_budget: float = 20.0) -> dict:
@@ -116,7 +119,7 @@ def main() -> int:
                     .to(torch.float16))
     comm = VirtualComm(world_size=WORLD, device=dev, buff_size_=BUFF_BYTES, nslots=NSLOTS,
                        waves_per_rank=WAVES_PER_RANK, threads_per_block=THREADS,
-                       placement=PLACEMENT)
+                       placement=PLACEMENT, cache_policy=CACHE_POLICY)
 
     def step():
         comm.run(lambda r: reducescatter(bufs[r], comm))
@@ -151,11 +154,13 @@ def main() -> int:
                                "x 256 MiB fp16 on one MI355X, in place",
                    "world": WORLD, "per_rank_bytes": PER_RANK_BYTES, "staging_per_rank": BUFF_BYTES,
                    "nslots": NSLOTS, "waves_per_rank": WAVES_PER_RANK, "threads": THREADS,
-                   "placement": ["spread", "local"][PLACEMENT], "grid_blocks": comm.last_grid,
+                   "placement": ["spread", "local"][PLACEMENT],
+                   "staging_cache_policy": ["agent", "system", "xcd-local"][CACHE_POLICY],
+                   "grid_blocks": comm.last_grid,
                    "payload_bytes_per_step": payload},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH},
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(CACHE_POLICY)},
         "kernel_ms": round(kernel_ms, 4),
         "copy_bw_gbps": round(copy_gbps, 1),
         "frac_of_copy_bw": round(achieved / copy_gbps, 4),

@@ -166,7 +166,10 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
         c = x / npos;
     }
     const int p = c / a.blocks_per_group;
-    const int w = (c % a.blocks_per_group) * (int)(blockDim.x >> 6) + wave_in_block();
+    // the wave index is the same in every lane: keep it (and all the index
+    // arithmetic that hangs off it) in scalar registers
+    const int w = (c % a.blocks_per_group) * (int)(blockDim.x >> 6) +
+                  (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     if (w >= a.waves) return;
     if (CPI == 2 && xcc_id() != x % kXcds) {
         // the XCD-local policy rests on block x running on XCD x % 8
@@ -207,20 +210,34 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
     const uint64_t t_begin = timing ? wall_clock64() : 0;
 
-    // Block indices of group n: U blocks of this wave-channel inside step n / groups_per_step.
-    struct Group { uint32_t step, idx[U], g[U]; bool valid[U], first, last; };
-    auto group_of = [&](uint32_t n) {
-        Group q;
-        q.step = n / groups_per_step;
-        const uint32_t k0 = (n % groups_per_step) * (uint32_t)U;
-        q.first = k0 == 0;
-        q.last = k0 + (uint32_t)U >= K;
+    // Group = U blocks of this wave-channel inside one step.  The walk over
+    // (step, first block) is kept incrementally: no division in the loop.
+    struct Group { uint32_t step, slot, k0, idx[U], g[U]; bool valid[U], first, last; };
+    auto fill = [&](Group& q) {
+        q.first = q.k0 == 0;
+        q.last = q.k0 + (uint32_t)U >= K;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            q.idx[u] = (k0 + (uint32_t)u) * W + (uint32_t)w;
+            q.idx[u] = (q.k0 + (uint32_t)u) * W + (uint32_t)w;
             q.g[u] = q.step * a.step_blocks + q.idx[u];
             q.valid[u] = q.g[u] < a.nblocks;
         }
+    };
+    auto first_group = [&]() {
+        Group q;
+        q.step = 0; q.slot = 0; q.k0 = 0;
+        fill(q);
+        return q;
+    };
+    auto next_group = [&](const Group& cur) {
+        Group q;
+        q.step = cur.step; q.slot = cur.slot; q.k0 = cur.k0 + (uint32_t)U;
+        if (q.k0 >= K) {
+            q.k0 = 0;
+            ++q.step;
+            q.slot = cur.slot + 1 == a.nslots ? 0 : cur.slot + 1;
+        }
+        fill(q);
         return q;
     };
     // load_ll128 of the wave's own rows for one group.
@@ -250,12 +267,13 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     u32x4 v[U], vnext[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
-    if (role.load && ngroups) load_own(group_of(0), v);
+    Group q = first_group();
+    if (role.load && ngroups) load_own(q, v);
 
     for (uint32_t n = 0; n < ngroups; ++n) {
-        const Group q = group_of(n);
+        const Group qn = next_group(q);
         const uint32_t s = q.step;
-        const uint32_t slot_off = (s % a.nslots) * a.slot_bytes + (uint32_t)p * a.step_msg;
+        const uint32_t slot_off = q.slot * a.slot_bytes + (uint32_t)p * a.step_msg;
         const uint32_t tag = (a.epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the credit for the slot this step
         // goes into is only needed before the send, so its load is issued
@@ -282,7 +300,7 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
                 if (q.valid[u])
                     r[u] = ld128<LDCP>(own, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u);
         }
-        if (role.load && n + 1 < ngroups) load_own(group_of(n + 1), vnext);
+        if (role.load && n + 1 < ngroups) load_own(qn, vnext);
         if (role.recv && PROTO == PROTO_LL128) {
             uint32_t pending = 0;
 #pragma unroll
@@ -361,6 +379,7 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = vnext[u];
+        q = qn;
     }
     if (timing && lane_id() == 0) {
         unsigned long long* st = reinterpret_cast<unsigned long long*>(a.stats) + 8 * h;
