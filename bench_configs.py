@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Throughput of the other BASELINE.json configurations on one MI355X (bench.py
+covers the headline).  One JSON line per measurement; every case is also
+checked for correctness (bit-exact copies; reductions against the device
+adder folded in ring order).
+
+    python bench_configs.py [--quick]
+
+  config 2  sendrecv 256 MiB fp16, rank 0 -> rank 1: LL128, Simple, direct copy
+  config 3  ring broadcast 64 MiB, 8 ranks, 8 x 512 KiB slots
+  config 4  ring reduce and reducescatter, 32 Mi elements per rank, f16 / bf16 / f32
+  config 5  ring allgather sweep, shard 512 B .. 128 MiB, LL128 vs Simple
+
+Algorithmic bytes: copy 2S; sendrecv over h hops
+(2 + 2h) S; broadcast / allgather (3N - 2) S; reduce / reducescatter (3N + 1) S.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+from mintccl_amd import _lib, primitive, sendrecv_buffer, sendrecv_direct  # noqa: E402
+from mintccl_amd.allgather import allgather  # noqa: E402
+from mintccl_amd.broadcast import broadcast  # noqa: E402
+from mintccl_amd.common import VirtualComm  # noqa: E402
+from mintccl_amd.reduce import reduce  # noqa: E402
+from mintccl_amd.reducescatter import reducescatter  # noqa: E402
+
+DEV = torch.device("cuda:0")
+TDT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+
+
+def time_ms(fn, reps: int) -> float:
+    """Average device time of `reps` back-to-back launches (the host side of a
+    launch hides behind the previous kernel)."""
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def emit(**kw) -> None:
+    print(json.dumps(kw), flush=True)
+
+
+def comm_for(world: int, proto: int, slots=None, **kw) -> VirtualComm:
+    """slots = (nslots, slot_bytes) for the geometry BASELINE.json names;
+    None = the library's tuned default."""
+    if slots is not None:
+        kw.update(buff_size_=slots[0] * slots[1], nslots=slots[0])
+    return VirtualComm(world_size=world, device=DEV, protocol=proto, **kw)
+
+
+def config2(reps: int) -> None:
+    n = 134217728
+    g = torch.Generator(device=DEV).manual_seed(1)
+    src = torch.randn(n, generator=g, device=DEV, dtype=torch.float32).to(torch.float16)
+    dst = torch.zeros_like(src)
+    S = n * 2
+    for name, proto in (("ll128", 0), ("simple", 1)):
+        for label, slots in (("8x512KiB", (8, 512 * 1024)), ("tuned", None)):
+            comm = comm_for(2, proto, slots, waves_per_rank=512 if slots else None)
+
+            def step():
+                with comm.rank(0):
+                    sendrecv_buffer.send(src, 1, comm)
+                with comm.rank(1):
+                    sendrecv_buffer.recv(dst, 0, comm)
+                sendrecv_buffer.sync(comm)
+
+            dst.zero_()
+            step()
+            comm.check()
+            ok = torch.equal(dst.view(torch.int16), src.view(torch.int16))
+            ms = time_ms(step, reps)
+            emit(config=2, op="sendrecv", protocol=name, staging=label, bytes=S, ms=round(ms, 4),
+                 alg_gbps=round(4 * S / ms / 1e6, 1), algbw_gbps=round(S / ms / 1e6, 1), ok=ok,
+                 grid=comm.last_grid)
+    comm = VirtualComm(world_size=2, device=DEV)
+
+    def direct():
+        with comm.rank(0):
+            sendrecv_direct.send(src, 1, comm)
+        with comm.rank(1):
+            sendrecv_direct.recv(dst, 0, profile=False, comm=comm)
+
+    dst.zero_()
+    direct()
+    torch.cuda.synchronize()
+    ok = torch.equal(dst.view(torch.int16), src.view(torch.int16))
+    ms = time_ms(direct, reps)
+    emit(config=2, op="sendrecv_direct", protocol="simple copy", bytes=S, ms=round(ms, 4),
+         alg_gbps=round(2 * S / ms / 1e6, 1), algbw_gbps=round(S / ms / 1e6, 1), ok=ok)
+
+
+def config3(reps: int) -> None:
+    world, n = 8, 33554432
+    g = torch.Generator(device=DEV).manual_seed(2)
+    root = (torch.rand(n, generator=g, device=DEV) * 8 - 4).to(torch.float16)
+    bufs = [root.clone() if r == 0 else torch.zeros_like(root) for r in range(world)]
+    S = n * 2
+    for name, proto in (("ll128", 0), ("simple", 1)):
+        for label, slots in (("8x512KiB", (8, 512 * 1024)), ("tuned", None)):
+            comm = comm_for(world, proto, slots, waves_per_rank=512 if slots else None)
+            for b in bufs[1:]:
+                b.zero_()
+
+            def step():
+                comm.run(lambda r: broadcast(bufs[r], 0, comm))
+
+            step()
+            comm.check()
+            ok = all(torch.equal(b.view(torch.int16), root.view(torch.int16)) for b in bufs)
+            ms = time_ms(step, reps)
+            emit(config=3, op="broadcast", protocol=name, staging=label, world=world, bytes=S,
+                 ms=round(ms, 4), alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1),
+                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+
+
+def fold_device(rows: list, order: list[int]) -> torch.Tensor:
+    acc = rows[order[0]].clone()
+    for r in order[1:]:
+        acc = primitive.Sum(rows[r].contiguous(), acc)
+    return acc
+
+
+def config4(reps: int) -> None:
+    world, n_total = 8, 33554432
+    n = n_total // world
+    for dt in ("f16", "bf16", "f32"):
+        orig = []
+        for r in range(world):
+            g = torch.Generator(device=DEV).manual_seed(3000 + r)
+            orig.append(torch.randn(world, n, generator=g, device=DEV, dtype=torch.float32)
+                        .to(TDT[dt]))
+        S = n_total * orig[0].element_size()
+        for label, slots in (("8x1MiB", (8, 1 << 20)), ("tuned", None)):
+            comm = comm_for(world, 0, slots, waves_per_rank=512 if slots else None)
+            bufs = [o.clone() for o in orig]
+
+            def rs():
+                comm.run(lambda r: reducescatter(bufs[r], comm))
+
+            rs()
+            comm.check()
+            ok = all(torch.equal(bufs[c][c].view(torch.uint8),
+                                 fold_device([orig[r][c] for r in range(world)],
+                                             [(c + k) % world for k in range(world)]).view(torch.uint8))
+                     for c in range(world))
+            ms = time_ms(rs, reps)
+            emit(config=4, op="reducescatter", dtype=dt, staging=label, world=world, bytes=S,
+                 ms=round(ms, 4), alg_gbps=round((3 * world + 1) * S / ms / 1e6, 1),
+                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+            flat = [o.reshape(-1).clone() for o in orig]
+
+            def rd():
+                comm.run(lambda r: reduce(flat[r], 0, comm))
+
+            rd()
+            comm.check()
+            ok = torch.equal(flat[0].view(torch.uint8),
+                             fold_device([o.reshape(-1) for o in orig], list(range(world)))
+                             .view(torch.uint8))
+            ms = time_ms(rd, reps)
+            emit(config=4, op="reduce", dtype=dt, staging=label, world=world, bytes=S,
+                 ms=round(ms, 4), alg_gbps=round((3 * world + 1) * S / ms / 1e6, 1),
+                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+
+
+def config5(reps: int, max_log2: int) -> None:
+    world = 8
+    for name, proto in (("ll128", 0), ("simple", 1)):
+        comms = {"8x512KiB": comm_for(world, proto, (8, 512 * 1024), waves_per_rank=512),
+                 "tuned": comm_for(world, proto, None)}
+        for log2 in range(9, max_log2 + 1):
+            shard = 1 << log2
+            n = shard // 2
+            bufs = []
+            for r in range(world):
+                g = torch.Generator(device=DEV).manual_seed(4 + r)
+                b = torch.zeros(world, n, device=DEV, dtype=torch.float16)
+                b[r] = (torch.rand(n, generator=g, device=DEV) * 2 - 1).to(torch.float16)
+                bufs.append(b)
+            want = torch.stack([bufs[r][r] for r in range(world)])
+            for label, comm in comms.items():
+                def step():
+                    comm.run(lambda r: allgather(bufs[r], comm))
+
+                step()
+                comm.check()
+                ok = all(torch.equal(b.view(torch.int16), want.view(torch.int16)) for b in bufs)
+                # launch straight from a prepared descriptor: leaves out the
+                # per-rank Python bookkeeping, which would dominate small sizes
+                ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+                d = comm.make_op(_lib.OP_ALLGATHER, _lib.BYTES, shard, ptrs, ptrs,
+                                 list(range(world)) + [0], row_stride=shard)
+                ms = time_ms(lambda: comm.launch(d), (reps if log2 < 24 else max(2, reps // 2)) * 4)
+                comm.check()
+                S = world * shard
+                emit(config=5, op="allgather", protocol=name, staging=label, world=world,
+                     shard_bytes=shard, us=round(ms * 1e3, 2),
+                     alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1),
+                     busbw_gbps=round(shard * (world - 1) / ms / 1e6, 1), ok=ok)
+            del bufs
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
+    ap.add_argument("--only", type=int, default=0, help="run one config (2..5)")
+    args = ap.parse_args()
+    reps = 3 if args.quick else 8
+    torch.cuda.set_device(DEV)
+    if args.only in (0, 2):
+        config2(reps)
+    if args.only in (0, 3):
+        config3(reps)
+    if args.only in (0, 4):
+        config4(reps)
+    if args.only in (0, 5):
+        config5(reps, 24 if args.quick else 27)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -139,19 +139,37 @@ class VirtualComm:
         if not 1 <= self.world_size <= _lib.MAX_RANKS:
             raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
         self.device = torch.device(device)
-        self.buff_size = buff_size_ if buff_size_ is not None else buff_size()
-        self.nslots = nslots if nslots is not None else num_slots()
+        # Geometry.  Explicit arguments win, then the reference's MINTCCL_*
+        # knobs (common.py:85-101: NUM_BLOCKS x NUM_WARPS 32-lane warps per rank,
+        # BUFF_SIZE of staging).  With neither, the MI355X-tuned default is
+        # used: 3 slots of 512 KiB and 512 wave-channels per rank, every hop
+        # of a channel on one XCD and staging kept in that XCD's L2.
+        knobs = ("MINTCCL_NUM_BLOCKS", "MINTCCL_NUM_WARPS", "MINTCCL_BUFFSIZE", "MINTCCL_NSLOTS")
+        reference_geometry = any(os.getenv(k) for k in knobs)
+        tuned = not reference_geometry
+        if nslots is None:
+            nslots = num_slots() if (reference_geometry or buff_size_ is not None) else 3
+        if buff_size_ is None:
+            buff_size_ = buff_size() if reference_geometry else nslots * 512 * 1024
+        self.buff_size, self.nslots = buff_size_, nslots
         if self.buff_size % self.nslots:
             raise ValueError("MINTCCL_BUFFSIZE must be a multiple of MINTCCL_NSLOTS")
         self.slot_bytes = self.buff_size // self.nslots
         self.protocol = protocol if protocol is not None else protocol_env()
-        self.placement = placement if placement is not None else placement_env()
-        # reference geometry: NUM_BLOCKS blocks of NUM_WARPS 32-lane warps per rank
-        self.waves_per_rank = (waves_per_rank if waves_per_rank is not None
-                               else max(1, num_blocks() * num_warps() // 2))
+        if placement is None:
+            placement = placement_env() if os.getenv("MINTCCL_PLACEMENT") else (
+                _lib.PLACE_LOCAL if tuned else _lib.PLACE_SPREAD)
+        self.placement = placement
+        if waves_per_rank is None:
+            waves_per_rank = (max(1, num_blocks() * num_warps() // 2) if reference_geometry
+                              else 512)
+        self.waves_per_rank = waves_per_rank
         self.threads_per_block = (threads_per_block if threads_per_block is not None
                                   else _env_int("MINTCCL_THREADS", 256))
-        self.cache_policy = cache_policy if cache_policy is not None else cache_policy_env()
+        if cache_policy is None:
+            cache_policy = cache_policy_env() if os.getenv("MINTCCL_CACHE") else (
+                2 if self.placement == _lib.PLACE_LOCAL else 0)
+        self.cache_policy = cache_policy
         if self.cache_policy == 2 and self.placement != _lib.PLACE_LOCAL:
             raise ValueError("the XCD-local cache policy needs the local placement")
         self.spin_budget = spin_budget
@@ -245,6 +263,14 @@ class VirtualComm:
             step_blocks, max(1, self.waves_per_rank // pipes))
         d.threads_per_block = self.threads_per_block
         d.placement, d.cache_policy = self.placement, self.cache_policy
+        if self.placement == _lib.PLACE_LOCAL:
+            # whole channels are dealt to the 8 XCDs; when the channel count
+            # does not divide, this launch runs spread with agent-scope staging
+            wpb = max(1, min(self.threads_per_block // 64, d.waves_per_channel_group))
+            channels = pipes * -(-d.waves_per_channel_group // wpb)
+            if channels % 8:
+                d.placement = _lib.PLACE_SPREAD
+                d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
         d.debug_skip_origin = int(skip_origin)

@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "kernels.hpp"
 #include "ring.hpp"
 
@@ -179,11 +181,23 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
         default: kernel = ring_kernel<PROTO, DT, CP, 1>; break;
     }
     // Every wavefront of the launch polls words other wavefronts write, so
-    // the whole grid has to be resident at once.
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) != hipSuccess)
-        return MINT_ERR_HIP;
-    if (plan.blocks > per_cu * device_cus()) return MINT_ERR_RESIDENCY;
+    // the whole grid has to be resident at once.  The occupancy of a kernel
+    // at a block size does not change: ask once (per block size) and keep it.
+    // (these statics are per template instantiation, i.e. per kernel family)
+    static std::atomic<int> cached[3][9] = {};       // [unroll][threads / 64]
+    static std::atomic<int> cus{0};
+    std::atomic<int>& memo = cached[plan.unroll == 4 ? 2 : (plan.unroll == 2 ? 1 : 0)]
+                                   [plan.threads / 64];
+    int per_cu = memo.load(std::memory_order_relaxed);
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) !=
+            hipSuccess)
+            return MINT_ERR_HIP;
+        memo.store(per_cu, std::memory_order_relaxed);
+    }
+    int ncu = cus.load(std::memory_order_relaxed);
+    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
+    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
     hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
                        plan.args);
     return launch_status();

@@ -114,10 +114,10 @@ __device__ __forceinline__ bool aborted(const uint64_t* status) {
 // aborted.  (wait_ll128, protocol.py:161-180, with a bound.)
 __device__ __forceinline__ bool wait_count(const uint64_t* word, uint32_t epoch, uint32_t need,
                                            uint32_t& cached, uint32_t budget,
-                                           const uint64_t* status, bool acquire) {
+                                           const uint64_t* status) {
     if (cached >= need) return true;
     for (uint32_t spins = 0;; ++spins) {
-        uint64_t v = acquire ? ld64_acquire(word) : ld64_agent(word);
+        uint64_t v = ld64_agent(word);
         uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
         uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
         if (hi == epoch && lo >= need) { cached = lo; return true; }
@@ -284,7 +284,7 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
         if (ask_credit) credit_word = ld64_agent(nxt_tail);
         if (q.first && PROTO == PROTO_SIMPLE && role.recv) {
             const uint64_t t0 = timing ? wall_clock64() : 0;
-            if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status, true)) {
+            if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status)) {
                 report_timeout(a.status, p, h, w, s);
                 return;
             }
@@ -329,8 +329,8 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
             const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)credit_word);
             if (hi == a.epoch && lo >= need) {
                 credits_seen = lo;
-            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget, a.status,
-                                   false)) {
+            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
+                                   a.status)) {
                 report_timeout(a.status, p, h, w, s);
                 return;
             }
@@ -374,8 +374,15 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
                 if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
                 else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
             }
-            if (PROTO == PROTO_SIMPLE && role.send && lane_id() == 0)
-                st64_release(nxt_head, flag_hi | (uint64_t)(s + 1));
+            if (PROTO == PROTO_SIMPLE && role.send) {
+                // Simple protocol: data first, then the step counter.  The data
+                // loads of the receiver skip the L1 (LDCP), so no invalidate.
+                wait_stores_visible();
+                if (lane_id() == 0) {
+                    if (STCP == CP_NONE) st64_local(nxt_head, flag_hi | (uint64_t)(s + 1));
+                    else st64_agent(nxt_head, flag_hi | (uint64_t)(s + 1));
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = vnext[u];
