@@ -101,7 +101,12 @@ typedef struct {
     uint32_t spin_budget;  /* polls before a wait gives up; 0 = default */
     uint64_t status;       /* device address of MINT_STATUS_WORDS uint64 */
     uint32_t debug_skip_origin; /* testing: origin hop sends nothing */
-    uint32_t reserved;
+    uint32_t credit_offset; /* byte offset of the credit words inside each rank's
+                               staging; 0 = right after the slots.  A caller
+                               that changes slot geometry between launches on
+                               the same staging keeps this fixed (beyond its
+                               largest nslots * slot_bytes, multiple of 256) so
+                               that credit words and payload never share bytes */
     uint64_t debug_stats;  /* 0.  A library built with -DMINT_RING_STATS takes
                               the device address of (hops + 1) x 8 zeroed
                               uint64 and fills, per position, {groups,

@@ -51,7 +51,7 @@ class RingOp(ctypes.Structure):
         ("placement", ctypes.c_int32), ("cache_policy", ctypes.c_int32),
         ("flag_epoch", ctypes.c_uint32), ("spin_budget", ctypes.c_uint32),
         ("status", ctypes.c_uint64),
-        ("debug_skip_origin", ctypes.c_uint32), ("reserved", ctypes.c_uint32),
+        ("debug_skip_origin", ctypes.c_uint32), ("credit_offset", ctypes.c_uint32),
         ("debug_stats", ctypes.c_uint64),
     ]
 

@@ -103,6 +103,13 @@ class Timer:
         print(f"# {tag}time: {self.elapsed}s")
 
 
+# Tuned geometry for MI355X (measured): about 4600 wavefronts in flight in
+# total, one 1 KiB block per wave-channel per step, 3 slots; a slot may grow to
+# this many bytes when a collective has few pipelines and hops.
+TUNED_TOTAL_WAVES = 4608
+TUNED_SLOT_BUDGET = 2304 * 1024
+
+
 class RingTimeout(RuntimeError):
     """A bounded wait inside the ring kernel ran out (status word 0 == 1)."""
 
@@ -147,10 +154,14 @@ class VirtualComm:
         knobs = ("MINTCCL_NUM_BLOCKS", "MINTCCL_NUM_WARPS", "MINTCCL_BUFFSIZE", "MINTCCL_NSLOTS")
         reference_geometry = any(os.getenv(k) for k in knobs)
         tuned = not reference_geometry
+        # tuned mode sizes slots per collective (see make_op) inside a fixed
+        # budget of staging per rank
+        self.auto_geometry = (tuned and buff_size_ is None and nslots is None
+                              and waves_per_rank is None)
         if nslots is None:
             nslots = num_slots() if (reference_geometry or buff_size_ is not None) else 3
         if buff_size_ is None:
-            buff_size_ = buff_size() if reference_geometry else nslots * 512 * 1024
+            buff_size_ = buff_size() if reference_geometry else nslots * TUNED_SLOT_BUDGET
         self.buff_size, self.nslots = buff_size_, nslots
         if self.buff_size % self.nslots:
             raise ValueError("MINTCCL_BUFFSIZE must be a multiple of MINTCCL_NSLOTS")
@@ -176,6 +187,8 @@ class VirtualComm:
         self._lib = _lib.lib()          # fails loudly if the extension is missing
         # slots + credit words (never more than slot_bytes / 4), zeroed: flag 0
         # and credit 0 mean "nothing yet" (2_sendrecv_indirect.py:59-60).
+        if self.buff_size % 256:
+            raise ValueError("staging size must be a multiple of 256 bytes")
         self.rank_stride = self.buff_size + max(4096, self.slot_bytes // 4)
         self.rank_stride = (self.rank_stride + 255) // 256 * 256
         self.staging = torch.zeros(self.world_size * self.rank_stride, dtype=torch.uint8,
@@ -254,13 +267,26 @@ class VirtualComm:
             d.output[r] = outputs.get(r, NULL)
             d.staging[r] = self.staging_ptr(r)
         d.count_bytes, d.row_stride = count_bytes, row_stride
-        d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
+        # credit words at a fixed place, whatever slot geometry a launch uses
+        d.credit_offset = self.buff_size
         pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER) else 1
-        step_blocks = self.slot_bytes // 1024 // pipes
-        if self.slot_bytes % 1024 or step_blocks == 0:
-            raise ValueError("slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
-        d.waves_per_channel_group = _largest_divisor_at_most(
-            step_blocks, max(1, self.waves_per_rank // pipes))
+        if self.auto_geometry:
+            # spread the wavefront budget over (pipeline, hop) groups; one
+            # block per wave-channel per step; whole blocks of 4 waves per XCD
+            npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: self.world_size,
+                    _lib.OP_ALLGATHER: self.world_size}.get(op, self.world_size + 1)
+            waves = TUNED_TOTAL_WAVES // (pipes * npos) // 32 * 32
+            waves = max(32, min(waves, TUNED_SLOT_BUDGET // 1024 // pipes // 32 * 32))
+            d.slot_bytes, d.nslots = pipes * waves * 1024, self.nslots
+            d.waves_per_channel_group = waves
+        else:
+            d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
+            step_blocks = self.slot_bytes // 1024 // pipes
+            if self.slot_bytes % 1024 or step_blocks == 0:
+                raise ValueError(
+                    "slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
+            d.waves_per_channel_group = _largest_divisor_at_most(
+                step_blocks, max(1, self.waves_per_rank // pipes))
         d.threads_per_block = self.threads_per_block
         d.placement, d.cache_policy = self.placement, self.cache_policy
         if self.placement == _lib.PLACE_LOCAL:

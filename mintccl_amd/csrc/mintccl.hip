@@ -148,6 +148,10 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     a.steps = (a.nblocks + a.step_blocks - 1) / a.step_blocks;
     if (a.steps > kMaxSteps) return MINT_ERR_TOO_LARGE;
     a.credit_off = a.nslots * a.slot_bytes;
+    if (op->credit_offset) {
+        if (op->credit_offset < a.credit_off || op->credit_offset % 256) return MINT_ERR_GEOMETRY;
+        a.credit_off = op->credit_offset;
+    }
     a.epoch = op->flag_epoch;
     a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
     a.status = reinterpret_cast<uint64_t*>(op->status);

@@ -12,6 +12,7 @@ import torch
 from . import _lib
 from ._ops import check_buffer, comm_or_default, nbytes
 from .common import VirtualComm
+from .protocol import packed_bytes
 from .topology import find_route, uniform_topology
 
 _KEY = "sendrecv_buffer"
@@ -35,8 +36,8 @@ def recv(buff: torch.Tensor, peer: int, comm: VirtualComm | None = None) -> None
                             "count": nbytes(buff), "src": peer, "keep": buff}
 
 
-def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None, staging=None,
-            geometry=None) -> None:
+def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None,
+            full_size_staging: bool = False) -> None:
     # 3_sendrecv_buffer.py:111-113
     if s["dst"] != r["rank"] or r["src"] != s["rank"]:
         raise ValueError("send and recv do not name each other")
@@ -49,10 +50,19 @@ def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None, stagin
         raise ValueError(f"no route {s['rank']} -> {r['rank']}")
     d = comm.make_op(_lib.OP_SENDRECV, _lib.BYTES, s["count"], {s["rank"]: s["data_ptr"]},
                      {r["rank"]: r["data_ptr"]}, route, route_len=len(route))
-    if staging is not None:
-        for rank, ptr in staging.items():
-            d.staging[rank] = ptr
-        d.slot_bytes, d.nslots = geometry
+    if full_size_staging:
+        # every line of the message gets a slot of its own, so no hop ever
+        # waits for a credit (2_sendrecv_indirect.py:147-149); zeroed like the
+        # reference's, and kept alive until the next transfer replaces it,
+        # since the launch is asynchronous
+        slot = d.slot_bytes
+        d.nslots = max(1, -(-packed_bytes(s["count"]) // slot))
+        per_rank = d.nslots * slot + max(4096, slot // 4)
+        hops = torch.zeros(comm.world_size * per_rank, dtype=torch.uint8, device=comm.device)
+        comm._indirect_staging = hops
+        for k in range(comm.world_size):
+            d.staging[k] = hops.data_ptr() + k * per_rank
+        d.credit_offset = 0                      # right after this staging's own slots
     comm.launch(d)
 
 

@@ -91,6 +91,7 @@ def test_plan_geometry_without_a_gpu():
     # 8 pipelines x 9 positions x (16 waves / 4 per block)
     assert L.mint_ring_grid_blocks(d) == 8 * 9 * 4
     assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256
+    assert L.mint_ring_staging_bytes(make_op(credit_offset=8 << 20)) == (8 << 20) + 8 * 16 * 256
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES)) == 8 * 8 * 4
     d = make_op(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
     assert L.mint_ring_grid_blocks(d) == 8 * 32
@@ -105,6 +106,8 @@ def test_plan_geometry_without_a_gpu():
     (dict(flag_epoch=0), _lib.ERR_ARG), (dict(flag_epoch=4096), _lib.ERR_ARG),
     (dict(status=0), _lib.ERR_ARG), (dict(cache_policy=3), _lib.ERR_ARG),
     (dict(cache_policy=2, placement=0), _lib.ERR_ARG),   # XCD-local staging needs the local placement
+    (dict(credit_offset=4096), _lib.ERR_GEOMETRY),       # inside the slots
+    (dict(credit_offset=(4 << 20) + 100), _lib.ERR_GEOMETRY),
     (dict(debug_stats=0x1000), _lib.ERR_ARG),            # this build collects no wait accounting
     (dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, waves_per_channel_group=16),
      _lib.ERR_GEOMETRY),                                 # 4 channels cannot be dealt to 8 XCDs
