@@ -275,8 +275,12 @@ class VirtualComm:
             # block per wave-channel per step; whole blocks of 4 waves per XCD
             npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: self.world_size,
                     _lib.OP_ALLGATHER: self.world_size}.get(op, self.world_size + 1)
-            waves = TUNED_TOTAL_WAVES // (pipes * npos) // 32 * 32
-            waves = max(32, min(waves, TUNED_SLOT_BUDGET // 1024 // pipes // 32 * 32))
+            receivers = max(1, min(npos - 1, self.world_size))
+            # a slot of 512 KiB per 8 receiving ranks keeps the staging of an
+            # XCD's channels (3 slots x receivers / 8) inside its L2
+            slot_blocks = min(512 * max(1, 8 // receivers), TUNED_TOTAL_WAVES // npos,
+                              TUNED_SLOT_BUDGET // 1024)
+            waves = max(32, slot_blocks // pipes // 32 * 32)
             d.slot_bytes, d.nslots = pipes * waves * 1024, self.nslots
             d.waves_per_channel_group = waves
         else:

@@ -168,9 +168,19 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const int p = c / a.blocks_per_group;
     // the wave index is the same in every lane: keep it (and all the index
     // arithmetic that hangs off it) in scalar registers
-    const int w = (c % a.blocks_per_group) * (int)(blockDim.x >> 6) +
-                  (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
-    if (w >= a.waves) return;
+    const int wpb = (int)(blockDim.x >> 6);
+    const int gw = c % a.blocks_per_group;
+    const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
+    if (gw * wpb + wib >= a.waves) return;
+    // Index of this wave-channel inside its group: it decides which blocks of
+    // a step, which staging bytes and which credit word the wave owns.  Under
+    // the local placement the blocks of one XCD are numbered consecutively, so
+    // that what an XCD touches (staging, rows) is contiguous in memory instead
+    // of 4 KiB out of every 32: that spreads it over all channels and sets of
+    // that XCD's L2.
+    int w = gw * wpb + wib;
+    if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
+        w = (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
     if (CPI == 2 && xcc_id() != x % kXcds) {
         // the XCD-local policy rests on block x running on XCD x % 8
         report_error(a.status, 2, p, h, w, (uint64_t)xcc_id());

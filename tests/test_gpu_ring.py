@@ -217,6 +217,64 @@ def test_many_launches_reuse_staging_without_clearing(dev):
         assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
 
 
+def test_epoch_wraps_after_4095_launches(dev):
+    # sector tags carry 12 bits of epoch: the communicator clears staging when
+    # the counter wraps, so launch 4096 cannot be fooled by launch 1's lines
+    from mintccl_amd import _lib
+    from mintccl_amd.broadcast import broadcast
+    world, n = 4, 2048
+    comm = make_comm(world)
+    host = [torch.full((n,), float(r + 1), dtype=torch.float16) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    comm.run(lambda r: broadcast(bufs[r], 0, comm))
+    d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n * 2, {0: ptrs[0]},
+                     {r: ptrs[r] for r in range(1, world)}, [0, 1, 2, 3, 0], root=0)
+    for _ in range(_lib.MAX_EPOCH + 5):
+        comm.launch(d)
+    comm.check()
+    assert 1 <= comm.epoch <= 10
+    for r in range(world):
+        bufs[r].fill_(float(10 + r))
+    comm.run(lambda r: broadcast(bufs[r], 2, comm))
+    comm.check()
+    for b in bufs:
+        assert torch.all(b == 12.0)
+
+
+def test_payload_that_looks_like_credit_words_is_harmless(dev):
+    # collectives of different shapes use different slot sizes on the same
+    # staging memory; the credit words live at a fixed offset beyond every
+    # slot, so payload bytes are never read as credits.  The payload here is
+    # 64-bit words (epoch << 32 | huge count) for the epochs that follow.
+    from mintccl_amd import sendrecv_buffer
+    from mintccl_amd.broadcast import broadcast
+    world = 8
+    comm = make_comm(world)
+    n64 = 1 << 20
+    for round_ in range(3):
+        words = torch.arange(n64, dtype=torch.int64)
+        words = ((comm.epoch + 2 + (words % 3)) << 32) | 0x7FFFFFF0
+        src = words.to(dev)
+        dst = torch.zeros_like(src)
+        with comm.rank(0):
+            sendrecv_buffer.send(src, 1, comm)       # 2 positions: large slots
+        with comm.rank(1):
+            sendrecv_buffer.recv(dst, 0, comm)
+        sendrecv_buffer.sync(comm)
+        comm.check()
+        assert torch.equal(dst, src)
+        bufs = [src.clone() if r == 3 else torch.zeros_like(src) for r in range(world)]
+        comm.run(lambda r: broadcast(bufs[r], 3, comm))   # 8 positions: small slots
+        comm.check()
+        for b in bufs:
+            assert torch.equal(b, src)
+        host = rank_rows(world, 40000, "f16", seed0=round_)
+        rs = [h.to(dev) for h in host]
+        run_reducescatter(comm, rs)
+        assert same(rs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
+
 def test_a_lost_producer_times_out_instead_of_hanging(dev):
     from mintccl_amd import _lib
     from mintccl_amd.common import RingTimeout
