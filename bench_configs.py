@@ -10,6 +10,7 @@ adder folded in ring order).
   config 3  ring broadcast 64 MiB, 8 ranks, 8 x 512 KiB slots
   config 4  ring reduce and reducescatter, 32 Mi elements per rank, f16 / bf16 / f32
   config 5  ring allgather sweep, shard 512 B .. 128 MiB, LL128 vs Simple
+  next      ring allreduce (the reference's planned 8_allreduce), 64 and 256 MiB fp16
 
 Algorithmic bytes: copy 2S; sendrecv over h hops
 (2 + 2h) S; broadcast / allgather (3N - 2) S; reduce / reducescatter (3N + 1) S.
@@ -220,10 +221,48 @@ def config5(reps: int, max_log2: int) -> None:
             del bufs
 
 
+def allreduce_bench(reps: int) -> None:
+    """The reference's planned 8_allreduce: 8 ranks x 256 MiB fp16.  Payload
+    bytes (6N - 4) S: per chunk N own-row reads, 2N - 2 staging writes and
+    reads, N result writes."""
+    from mintccl_amd.allreduce import allreduce
+    world = 8
+    for n in (33554432, 134217728):
+        orig = []
+        for r in range(world):
+            g = torch.Generator(device=DEV).manual_seed(3000 + r)
+            orig.append(torch.randn(n, generator=g, device=DEV, dtype=torch.float32)
+                        .to(torch.float16))
+        S = n * 2
+        for name, proto in (("ll128", 0), ("simple", 1)):
+            comm = comm_for(world, proto, None)
+            bufs = [o.clone() for o in orig]
+
+            def step():
+                comm.run(lambda r: allreduce(bufs[r], comm))
+
+            step()
+            comm.check()
+            row = n // world
+            ok = True
+            for c in range(world):
+                want = fold_device([o[c * row:(c + 1) * row] for o in orig],
+                                   [(c + k) % world for k in range(world)])
+                ok = ok and all(torch.equal(b[c * row:(c + 1) * row].view(torch.int16),
+                                            want.view(torch.int16)) for b in bufs)
+            ms = time_ms(step, reps)
+            emit(config="next", op="allreduce", protocol=name, staging="tuned", world=world,
+                 bytes=S, ms=round(ms, 4), alg_gbps=round((6 * world - 4) * S / ms / 1e6, 1),
+                 algbw_gbps=round(S / ms / 1e6, 1),
+                 busbw_gbps=round(2 * (world - 1) / world * S / ms / 1e6, 1), ok=ok,
+                 grid=comm.last_grid)
+        del orig
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
-    ap.add_argument("--only", type=int, default=0, help="run one config (2..5)")
+    ap.add_argument("--only", type=int, default=0, help="run one config (2..5; 8 = allreduce)")
     args = ap.parse_args()
     reps = 3 if args.quick else 8
     torch.cuda.set_device(DEV)
@@ -235,6 +274,8 @@ def main() -> int:
         config4(reps)
     if args.only in (0, 5):
         config5(reps, 24 if args.quick else 27)
+    if args.only in (0, 8):
+        allreduce_bench(reps)
     return 0
 
 

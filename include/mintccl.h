@@ -51,7 +51,9 @@ typedef enum {
     MINT_OP_BROADCAST = 1,     /* 4_broadcast.py:27-76 */
     MINT_OP_REDUCE = 2,        /* 5_reduce.py:36-95 */
     MINT_OP_ALLGATHER = 3,     /* 6_allgather.py:79-138 (spatial variant) */
-    MINT_OP_REDUCESCATTER = 4  /* 7_reducescatter.py:13-79 */
+    MINT_OP_REDUCESCATTER = 4, /* 7_reducescatter.py:13-79 */
+    MINT_OP_ALLREDUCE = 5      /* the reference's planned 8_allreduce (README.md:23):
+                                  reducescatter and allgather in one pass round the ring */
 } mint_op;
 typedef enum {
     MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
@@ -83,11 +85,12 @@ typedef struct {
     uint64_t input[MINT_MAX_RANKS];   /* per rank; 0 = absent */
     uint64_t output[MINT_MAX_RANKS];  /* per rank; 0 = absent */
     uint64_t staging[MINT_MAX_RANKS]; /* per rank, mint_ring_staging_bytes() each */
-    uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE: bytes of the buffer;
-                              ALLGATHER/REDUCESCATTER: bytes of one row */
+    uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE: bytes of the
+                              buffer; ALLGATHER/REDUCESCATTER: bytes of one row */
     uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER: bytes between rows */
     uint32_t slot_bytes;   /* staging bytes of one step over all pipelines;
-                              multiple of 1024, >= 1024 per pipeline */
+                              multiple of 1024, >= 1024 per pipeline (per
+                              pipeline and phase for ALLREDUCE, which has 2) */
     uint32_t nslots;       /* slots in the circular staging buffer */
     uint32_t waves_per_channel_group; /* wave-channels per (pipeline, hop) */
     uint32_t threads_per_block;       /* multiple of 64 */

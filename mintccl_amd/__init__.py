@@ -9,6 +9,7 @@ Operator surface (same names and argument order as the reference scripts):
     reduce.reduce(buff, root)                   5_reduce.py
     allgather.allgather(buff)                   6_allgather.py
     reducescatter.reducescatter(buff)           7_reducescatter.py
+    allreduce.allreduce(buff)                   8_allreduce.py (planned there, README.md:23)
 
 plus ``common`` (knobs, ``VirtualComm``), ``primitive``, ``protocol`` and
 ``topology``.  All compute runs in ``libmintccl.so`` (hand-written HIP); the

@@ -269,13 +269,19 @@ class VirtualComm:
         d.count_bytes, d.row_stride = count_bytes, row_stride
         # credit words at a fixed place, whatever slot geometry a launch uses
         d.credit_offset = self.buff_size
-        pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER) else 1
+        pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER,
+                                          _lib.OP_ALLREDUCE) else 1
+        if op == _lib.OP_ALLREDUCE:
+            pipes *= 2            # a slot is shared by (pipeline, phase): two phases
         if self.auto_geometry:
             # spread the wavefront budget over (pipeline, hop) groups; one
             # block per wave-channel per step; whole blocks of 4 waves per XCD
             npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: self.world_size,
-                    _lib.OP_ALLGATHER: self.world_size}.get(op, self.world_size + 1)
+                    _lib.OP_ALLGATHER: self.world_size,
+                    _lib.OP_ALLREDUCE: 2 * self.world_size - 1}.get(op, self.world_size + 1)
             receivers = max(1, min(npos - 1, self.world_size))
+            if op == _lib.OP_ALLREDUCE:
+                npos = (npos + 1) // 2        # `pipes` already counts both phases
             # a slot of 512 KiB per 8 receiving ranks keeps the staging of an
             # XCD's channels (3 slots x receivers / 8) inside its L2
             slot_blocks = min(512 * max(1, 8 // receivers), TUNED_TOTAL_WAVES // npos,
@@ -297,7 +303,8 @@ class VirtualComm:
             # whole channels are dealt to the 8 XCDs; when the channel count
             # does not divide, this launch runs spread with agent-scope staging
             wpb = max(1, min(self.threads_per_block // 64, d.waves_per_channel_group))
-            channels = pipes * -(-d.waves_per_channel_group // wpb)
+            real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
+            channels = real_pipes * -(-d.waves_per_channel_group // wpb)
             if channels % 8:
                 d.placement = _lib.PLACE_SPREAD
                 d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy

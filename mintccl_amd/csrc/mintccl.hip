@@ -31,7 +31,9 @@ int device_cus() {
 
 int launch_status() { return hipGetLastError() == hipSuccess ? MINT_OK : MINT_ERR_HIP; }
 
-bool reducing(int op) { return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER; }
+bool reducing(int op) {
+    return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE;
+}
 
 // Everything the launch derives from the descriptor.
 struct Plan {
@@ -42,7 +44,7 @@ struct Plan {
 
 int make_plan(const mint_ring_op* op, Plan* plan) {
     if (!op || !plan) return MINT_ERR_ARG;
-    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_REDUCESCATTER) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLREDUCE) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
@@ -61,8 +63,10 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     a = RingArgs{};
     a.op = op->op;
     a.world = op->world;
-    const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER;
+    const bool allreduce = op->op == MINT_OP_ALLREDUCE;
+    const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER || allreduce;
     a.pipes = rowwise ? op->world : 1;
+    a.phases = allreduce ? 2 : 1;
 
     // ring / route
     bool seen[MINT_MAX_RANKS] = {};
@@ -93,27 +97,39 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
             break;
         }
         default:
-            a.hops = op->op == MINT_OP_ALLGATHER ? op->world - 1 : op->world;
+            a.hops = op->op == MINT_OP_ALLGATHER ? op->world - 1
+                     : allreduce                 ? 2 * op->world - 2
+                                                 : op->world;
             for (int p = 0; p < op->world; ++p) a.start[p] = (uint8_t)index_of(p);
     }
 
-    a.row_bytes = op->count_bytes;
-    a.row_stride = rowwise ? op->row_stride : 0;
-    plan->empty = op->count_bytes == 0 || op->world == 1 ||
-                  (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);
-    if (rowwise && (op->row_stride < op->count_bytes || !aligned16(op->row_stride)))
-        return MINT_ERR_ALIGN;
     const int dt_size = op->dtype == MINT_F32 ? 4 : (op->dtype == MINT_BYTES ? 1 : 2);
     if (op->count_bytes % dt_size) return MINT_ERR_ARG;
+    if (allreduce) {
+        // one buffer of count_bytes per rank, cut into `world` rows of whole
+        // 16-byte vectors; the last rows may be short or empty
+        const uint64_t per = (op->count_bytes + op->world - 1) / op->world;
+        a.row_bytes = (per + 15) / 16 * 16;
+        a.row_stride = a.row_bytes;
+        a.total_bytes = op->count_bytes;
+    } else {
+        a.row_bytes = op->count_bytes;
+        a.row_stride = rowwise ? op->row_stride : 0;
+        if (rowwise && (op->row_stride < op->count_bytes || !aligned16(op->row_stride)))
+            return MINT_ERR_ALIGN;
+    }
+    plan->empty = op->count_bytes == 0 || op->world == 1 ||
+                  (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);
 
     // which ranks need which buffers
     for (int p = 0; p < a.pipes && !plan->empty; ++p) {
         for (int h = 0; h <= a.hops; ++h) {
             const int rank = a.cyc[(a.start[p] + h) % a.cyc_len];
             const bool origin = h == 0, sink = h == a.hops;
-            const bool load = origin || (reducing(op->op) && !sink);
-            const bool save = sink || ((op->op == MINT_OP_BROADCAST ||
-                                        op->op == MINT_OP_ALLGATHER) && !origin);
+            const bool load = allreduce ? h < op->world : origin || (reducing(op->op) && !sink);
+            const bool save = allreduce ? h >= op->world - 1
+                                        : sink || ((op->op == MINT_OP_BROADCAST ||
+                                                    op->op == MINT_OP_ALLGATHER) && !origin);
             if (load && (!op->input[rank] || !aligned16(op->input[rank])))
                 return op->input[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
             if (save && (!op->output[rank] || !aligned16(op->output[rank])))
@@ -134,7 +150,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     // a slot is shared evenly by the pipelines, in whole 1 KiB blocks; what
     // does not divide is left unused
     if (op->slot_bytes % kBlockMsg) return MINT_ERR_GEOMETRY;
-    a.step_blocks = op->slot_bytes / kBlockMsg / (uint32_t)a.pipes;
+    a.step_blocks = op->slot_bytes / kBlockMsg / (uint32_t)(a.pipes * a.phases);
     if (a.step_blocks == 0) return MINT_ERR_GEOMETRY;
     a.step_msg = a.step_blocks * kBlockMsg;
     if (op->waves_per_channel_group == 0 || a.step_blocks % op->waves_per_channel_group)
@@ -142,7 +158,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     a.waves = (int)op->waves_per_channel_group;
     a.k_per_wave = a.step_blocks / (uint32_t)a.waves;
     const uint32_t raw_per_block = op->protocol == MINT_PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
-    const uint64_t nblocks = (op->count_bytes + raw_per_block - 1) / raw_per_block;
+    const uint64_t nblocks = (a.row_bytes + raw_per_block - 1) / raw_per_block;
     if (nblocks >= (1ull << 28)) return MINT_ERR_TOO_LARGE;
     a.nblocks = (uint32_t)nblocks;
     a.steps = (a.nblocks + a.step_blocks - 1) / a.step_blocks;
@@ -382,7 +398,8 @@ size_t mint_ring_staging_bytes(const mint_ring_op* op) {
     Plan plan;
     if (make_plan(op, &plan) != MINT_OK) return 0;
     return (size_t)plan.args.credit_off +
-           (size_t)plan.args.pipes * (size_t)plan.args.waves * kCreditStride;
+           (size_t)plan.args.pipes * (size_t)plan.args.phases * (size_t)plan.args.waves *
+               kCreditStride;
 }
 
 int mint_ring_grid_blocks(const mint_ring_op* op) {

@@ -14,7 +14,9 @@
 // occupies both position 0 and the last position (the reference lets the root
 // run both roles in one thread with a lag of `world_size` rounds,
 // 5_reduce.py:79-89, 7_reducescatter.py:57-67; here they are different
-// wavefronts, so nothing has to lag).
+// wavefronts, so nothing has to lag).  Allreduce is the same walk carried on:
+// 2 * world - 1 positions, the first `world` add, the rest copy, and every
+// position from the last adder on keeps the result.
 //
 // Each (pipeline, position) is served by W *wave-channels*; wave-channel w of
 // position h talks only to wave-channel w of positions h-1 and h+1.  Staging
@@ -36,7 +38,7 @@
 namespace mint {
 
 enum : int { OP_SENDRECV = 0, OP_BROADCAST = 1, OP_REDUCE = 2, OP_ALLGATHER = 3,
-             OP_REDUCESCATTER = 4 };
+             OP_REDUCESCATTER = 4, OP_ALLREDUCE = 5 };
 enum : int { PROTO_LL128 = 0, PROTO_SIMPLE = 1 };
 enum : int { PLACE_SPREAD = 0, PLACE_LOCAL = 1 };
 
@@ -54,10 +56,12 @@ struct RingArgs {
     uint8_t start[kMaxRanks];             // per pipeline: index of its root in cyc
     uint64_t input[kMaxRanks], output[kMaxRanks], staging[kMaxRanks];
     uint64_t row_bytes, row_stride;
+    uint64_t total_bytes;                 // 0, or clip row p to total_bytes - p * row_stride
+    int32_t phases;                       // staging shares per pipeline (2 for allreduce)
     uint32_t nblocks;                     // blocks per row
     uint32_t steps;                       // steps per row
     uint32_t slot_bytes, nslots;
-    uint32_t step_msg;                    // slot_bytes / pipes
+    uint32_t step_msg;                    // bytes of one share: slot_bytes / (pipes * phases)
     uint32_t step_blocks;                 // step_msg / 1024
     uint32_t k_per_wave;                  // step_blocks / waves
     uint32_t credit_off;                  // offset of the credit words in staging
@@ -78,10 +82,20 @@ __device__ __forceinline__ Role role_of(const RingArgs& a, int p, int h) {
     r.rank = a.cyc[(s + h) % a.cyc_len];
     r.next = a.cyc[(s + h + 1) % a.cyc_len];
     const bool origin = h == 0, sink = h == a.hops;
-    const bool reducing = a.op == OP_REDUCE || a.op == OP_REDUCESCATTER;
-    const bool copying_all = a.op == OP_BROADCAST || a.op == OP_ALLGATHER;
     r.recv = !origin;
     r.send = !sink;
+    if (a.op == OP_ALLREDUCE) {
+        // reduce-scatter then all-gather in one pass around the ring: the
+        // first `world` positions add (the last of them holds the finished
+        // sum and keeps a copy), the rest copy and forward
+        const bool adding = h < a.world;
+        r.load = adding;
+        r.reduce = adding && !origin;
+        r.save = h >= a.world - 1;
+        return r;
+    }
+    const bool reducing = a.op == OP_REDUCE || a.op == OP_REDUCESCATTER;
+    const bool copying_all = a.op == OP_BROADCAST || a.op == OP_ALLGATHER;
     r.load = origin || (reducing && !sink);
     r.reduce = reducing && !origin && !sink;
     r.save = sink || (copying_all && !origin);
@@ -191,18 +205,33 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
 
     const LaneMap m;
     const uint64_t row_off = (uint64_t)p * a.row_stride;
+    // allreduce splits one buffer into `world` rows; the last ones may be short or empty
+    uint64_t row_bytes = a.row_bytes;
+    uint32_t nblocks = a.nblocks;
+    if (a.total_bytes) {
+        const uint64_t left = a.total_bytes > row_off ? a.total_bytes - row_off : 0;
+        row_bytes = left < a.row_bytes ? left : a.row_bytes;
+        const uint32_t per_block = PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
+        nblocks = (uint32_t)((row_bytes + per_block - 1) / per_block);
+    }
     const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
     uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
 #if defined(MINT_RAW_LD_CP) || defined(MINT_RAW_ST_CP)
-    const Window in_w(in_row, (uint32_t)a.row_bytes), out_w(out_row, (uint32_t)a.row_bytes);
+    const Window in_w(in_row, (uint32_t)row_bytes), out_w(out_row, (uint32_t)row_bytes);
 #endif
     const uint32_t ring_bytes = a.nslots * a.slot_bytes;
     const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
     const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);
-    const uint32_t chan_off = a.credit_off + ((uint32_t)p * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
-    uint64_t* own_tail = reinterpret_cast<uint64_t*>(a.staging[role.rank] + chan_off);
+    // a rank can receive twice in one pipeline of an allreduce (once while
+    // the sum is built, once while it is handed round): each phase has its own
+    // share of the slots and its own credit words
+    const uint32_t share_recv = (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
+    const uint32_t share_send = (uint32_t)p * (uint32_t)a.phases + (h + 1 >= a.world && a.phases > 1 ? 1u : 0u);
+    const uint32_t own_chan = a.credit_off + (share_recv * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
+    const uint32_t nxt_chan = a.credit_off + (share_send * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
+    uint64_t* own_tail = reinterpret_cast<uint64_t*>(a.staging[role.rank] + own_chan);
     uint64_t* own_head = own_tail + 16;
-    uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + chan_off);
+    uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + nxt_chan);
     uint64_t* nxt_head = nxt_tail + 16;
 
     const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
@@ -230,7 +259,7 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
         for (int u = 0; u < U; ++u) {
             q.idx[u] = (q.k0 + (uint32_t)u) * W + (uint32_t)w;
             q.g[u] = q.step * a.step_blocks + q.idx[u];
-            q.valid[u] = q.g[u] < a.nblocks;
+            q.valid[u] = q.g[u] < nblocks;
         }
     };
     auto first_group = [&]() {
@@ -258,14 +287,14 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
             if (!q.valid[u]) continue;
             if (PROTO == PROTO_LL128) {
 #ifdef MINT_RAW_LD_CP
-                v[u] = ll_load_raw_w<MINT_RAW_LD_CP>(in_w, in_row, a.row_bytes, q.g[u], m);
+                v[u] = ll_load_raw_w<MINT_RAW_LD_CP>(in_w, in_row, row_bytes, q.g[u], m);
 #else
-                v[u] = ll_load_raw(in_row, a.row_bytes, q.g[u], m);
+                v[u] = ll_load_raw(in_row, row_bytes, q.g[u], m);
 #endif
             } else {
                 const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                v[u] = off + 16u <= a.row_bytes ? ld128_stream(in_row + off)
-                                               : load_guarded(in_row, off, 16u, a.row_bytes);
+                v[u] = off + 16u <= row_bytes ? ld128_stream(in_row + off)
+                                               : load_guarded(in_row, off, 16u, row_bytes);
             }
         }
     };
@@ -283,7 +312,8 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     for (uint32_t n = 0; n < ngroups; ++n) {
         const Group qn = next_group(q);
         const uint32_t s = q.step;
-        const uint32_t slot_off = q.slot * a.slot_bytes + (uint32_t)p * a.step_msg;
+        const uint32_t slot_off = q.slot * a.slot_bytes + share_recv * a.step_msg;
+        const uint32_t send_off = q.slot * a.slot_bytes + share_send * a.step_msg;
         const uint32_t tag = (a.epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the credit for the slot this step
         // goes into is only needed before the send, so its load is issued
@@ -359,21 +389,21 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
             if (role.save) {
                 if (PROTO == PROTO_LL128) {
 #ifdef MINT_RAW_ST_CP
-                    ll_save_raw_w<MINT_RAW_ST_CP>(out_w, out_row, a.row_bytes, q.g[u], m, v[u]);
+                    ll_save_raw_w<MINT_RAW_ST_CP>(out_w, out_row, row_bytes, q.g[u], m, v[u]);
 #else
-                    ll_save_raw(out_row, a.row_bytes, q.g[u], m, v[u]);
+                    ll_save_raw(out_row, row_bytes, q.g[u], m, v[u]);
 #endif
                 } else {
                     const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                    if (off + 16u <= a.row_bytes) st128_stream(out_row + off, v[u]);
-                    else store_guarded(out_row, off, 16u, a.row_bytes, v[u]);
+                    if (off + 16u <= row_bytes) st128_stream(out_row + off, v[u]);
+                    else store_guarded(out_row, off, 16u, row_bytes, v[u]);
                 }
             }
             if (role.send) {
                 if (PROTO == PROTO_LL128)
-                    ll_send<STCP>(nxt, slot_off + q.idx[u] * kBlockMsg, v[u], tag, m);
+                    ll_send<STCP>(nxt, send_off + q.idx[u] * kBlockMsg, v[u], tag, m);
                 else
-                    st128<STCP>(nxt, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
+                    st128<STCP>(nxt, send_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
             }
         }
         if (q.last) {

@@ -152,6 +152,30 @@ def allgather(xs: list) -> list:
     return [o.reshape(-1) for o in out]
 
 
+def allreduce_row_bytes(nbytes: int, world: int) -> int:
+    """Bytes of one chunk: the buffer is cut into ``world`` rows of whole
+    16-byte vectors; the last rows may be short or empty."""
+    return (-(-nbytes // world) + 15) // 16 * 16
+
+
+def allreduce(xs: list, dtype: str, ring: list[int] | None = None) -> list:
+    """Chunk c is folded in ring order starting from rank c's own value
+    (the reduce-scatter order) and every rank ends up with every folded chunk.
+    The reference only plans this collective (``README.md:23``); the order is
+    the one its reduce-scatter uses."""
+    n_ranks = len(xs)
+    ring = ring or identity_ring(n_ranks)
+    raw = [_bytes(x) for x in xs]
+    total = raw[0].size
+    row = allreduce_row_bytes(total, n_ranks)
+    out = np.empty(total, dtype=np.uint8)
+    for c in range(n_ranks):
+        lo, hi = min(c * row, total), min((c + 1) * row, total)
+        if hi > lo:
+            out[lo:hi] = fold([r[lo:hi] for r in raw], fold_order(ring, c), dtype)
+    return [out.copy() for _ in xs]
+
+
 def broadcast(xs: list, root: int) -> list:
     return [_bytes(xs[root]).copy() for _ in xs]
 

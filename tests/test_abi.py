@@ -97,11 +97,17 @@ def test_plan_geometry_without_a_gpu():
     assert L.mint_ring_grid_blocks(d) == 8 * 32
     d = make_op(op=_lib.OP_REDUCE, waves_per_channel_group=128, root=3)
     assert L.mint_ring_grid_blocks(d) == 9 * 32
+    # allreduce: 8 pipelines x 15 positions, two phases share a slot
+    d = make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=16, count_bytes=8 << 20)
+    assert L.mint_ring_grid_blocks(d) == 8 * 15 * 4
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 2 * 16 * 256
+    assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=64)) \
+        == _lib.ERR_GEOMETRY          # 512 KiB slot / 16 shares = 32 blocks per step
 
 
 @pytest.mark.parametrize("kw,err", [
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
-    (dict(op=7), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=6), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
     (dict(dtype=_lib.BYTES), _lib.ERR_ARG),          # a reduction needs a real dtype
     (dict(flag_epoch=0), _lib.ERR_ARG), (dict(flag_epoch=4096), _lib.ERR_ARG),
     (dict(status=0), _lib.ERR_ARG), (dict(cache_policy=3), _lib.ERR_ARG),

@@ -177,6 +177,53 @@ def test_xcd_local_policy_needs_local_placement(dev):
         make_comm(8, placement=0, cache_policy=2)
 
 
+def run_allreduce(comm, bufs):
+    from mintccl_amd.allreduce import allreduce
+    comm.run(lambda r: allreduce(bufs[r], comm))
+    comm.check()
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("n", [1, 7, 8, 63, 64, 4000, 100003, (1 << 20) + 9])
+def test_allreduce_f16(dev, world, n):
+    # ragged sizes: with few elements some chunks are short or empty
+    host = [normal(n, 3000 + r) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    run_allreduce(comm, bufs)
+    want = ring.allreduce([as_bytes(h) for h in host], "f16")
+    assert same(bufs, want)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f32"])
+@pytest.mark.parametrize("proto,place,cp", [(0, 0, 0), (1, 0, 0), (0, 1, 2), (1, 1, 2)])
+def test_allreduce_dtypes_protocols_policies(dev, dt, proto, place, cp):
+    world, n = 8, 300001
+    host = [normal(n, 3000 + r, TORCH_DT[dt]) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, protocol=proto, placement=place, cache_policy=cp,
+                     buff_size_=3 * 1024 * 1024, nslots=3, waves_per_rank=512)
+    run_allreduce(comm, bufs)
+    assert same(bufs, ring.allreduce([as_bytes(h) for h in host], dt))
+
+
+def test_allreduce_256mib_against_device_fold(dev):
+    from mintccl_amd import primitive
+    world, n = 8, 33554432          # 64 MiB per rank
+    g = torch.Generator(device=dev).manual_seed(11)
+    bufs = [torch.randn(n, generator=g, device=dev, dtype=torch.float16) for _ in range(world)]
+    orig = [b.clone() for b in bufs]
+    comm = make_comm(world)
+    run_allreduce(comm, bufs)
+    row = n // world
+    for c in range(world):
+        acc = orig[c][c * row:(c + 1) * row].clone()
+        for k in range(1, world):
+            acc = primitive.Sum(orig[(c + k) % world][c * row:(c + 1) * row].contiguous(), acc)
+        for r in range(world):
+            assert torch.equal(bufs[r][c * row:(c + 1) * row].view(torch.int16), acc.view(torch.int16))
+
+
 def test_permuted_ring(dev):
     # a non-uniform topology whose best ring is not the identity
     from mintccl_amd.topology import find_ring

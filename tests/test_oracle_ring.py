@@ -193,3 +193,27 @@ def test_copy_collectives_are_identities():
         for c in range(world):
             if r != c:      # only row r of rank r changes
                 assert (rs[r].reshape(world, n)[c] == rows[r].reshape(world, n)[c]).all()
+
+
+def test_allreduce_chunks_and_order():
+    # 4 ranks, 20 f16 values: rows of 16 bytes (8 values): chunks [0:8], [8:16], [16:20], []
+    assert ring.allreduce_row_bytes(40, 4) == 16
+    rows = [[2048.0, 1.0, 2048.0, 1.0], [1.0, 1.0, 1.0, 1.0], [1.0, 2048.0, 1.0, 2048.0],
+            [1.0, 1.0, 1.0, 1.0]]
+    xs = []
+    for r in range(4):
+        v = np.ones(20, dtype=np.float16)
+        v[0:8] = rows[r][0]; v[8:16] = rows[r][1]; v[16:20] = rows[r][2]
+        xs.append(v.view(np.uint8))
+    out = ring.allreduce(xs, "f16")
+    got = out[0].view(np.float16)
+    assert got[0] == 2048.0 and got[8] == 2048.0 and got[16] == 2052.0   # same hand values as reducescatter
+    assert all((o == out[0]).all() for o in out)
+    # against reducescatter + allgather of the padded buffer
+    world, n = 3, 1000
+    rng = np.random.default_rng(0)
+    xs = [rng.standard_normal(n).astype(np.float16).view(np.uint8) for _ in range(world)]
+    row = ring.allreduce_row_bytes(2 * n, world)
+    padded = [np.concatenate([x, np.zeros(world * row - x.size, np.uint8)]) for x in xs]
+    want = ring.allgather(ring.reducescatter(padded, "f16"))[0][:2 * n]
+    assert all((o == want).all() for o in ring.allreduce(xs, "f16"))
