@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0
 # the same counters' reading for a plain copy of known size; None until measured
 TRAFFIC_BYTES_PER_LAUNCH = {2: 2.931e9, 0: 7.780e9}
 
-# launch geometry used for the headline (DESIGN.md section 7): 3 slots of
+# launch geometry used for the headline: 3 slots of
 # 512 KiB per rank so that all staging of an XCD's channels stays in its 4 MiB
 # L2, 64 wave-channels per (chunk, hop), every hop of a channel on one XCD
 BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 3 * 512 * 1024))

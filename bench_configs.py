@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Throughput of the other BASELINE.json configurations on one MI355X (bench.py
+"""Throughput of the other benchmark configurations on one MI355X (bench.py
 covers the headline).  One JSON line per measurement; every case is also
 checked for correctness (bit-exact copies; reductions against the device
 adder folded in ring order).
@@ -12,7 +12,7 @@ adder folded in ring order).
   config 5  ring allgather sweep, shard 512 B .. 128 MiB, LL128 vs Simple
   next      ring allreduce (the reference's planned 8_allreduce), 64 and 256 MiB fp16
 
-Algorithmic bytes (DESIGN.md section 5): copy 2S; sendrecv over h hops
+Algorithmic bytes: copy 2S; sendrecv over h hops
 (2 + 2h) S; broadcast / allgather (3N - 2) S; reduce / reducescatter (3N + 1) S.
 """
 from __future__ import annotations
@@ -61,7 +61,7 @@ def emit(**kw) -> None:
 
 
 def comm_for(world: int, proto: int, slots=None, **kw) -> VirtualComm:
-    """slots = (nslots, slot_bytes) for the geometry BASELINE.json names;
+    """slots = (nslots, slot_bytes) for the geometry the configuration names;
     None = the library's tuned default."""
     if slots is not None:
         kw.update(buff_size_=slots[0] * slots[1], nslots=slots[0])

@@ -1,5 +1,5 @@
-"""Seeded inputs shared by the CPU and GPU tests (the configurations named in
-BASELINE.json, generated on the CPU so oracle and device see the same bits)."""
+"""Seeded inputs shared by the CPU and GPU tests (the five benchmark
+configurations, generated on the CPU so oracle and device see the same bits)."""
 from __future__ import annotations
 
 import numpy as np

@@ -84,7 +84,7 @@ def test_unpack_counts_wrong_flags(dev, layout):
 @pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
 @pytest.mark.parametrize("stride", [1, 0])
 def test_config1_roundtrip_on_device(dev, layout, stride):
-    # BASELINE config 1 on the GPU: 1 MiB fp16 uniform[-1,1] seed 0
+    # benchmark configuration 1 on the GPU: 1 MiB fp16 uniform[-1,1] seed 0
     from mintccl_amd import protocol
     x = uniform(524288, -1.0, 1.0, 0)
     d = x.to(dev)

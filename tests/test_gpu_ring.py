@@ -384,7 +384,7 @@ def test_one_flag_per_128_byte_line_is_not_enough(lib, dev):
     print(f"lines checked {checked}, torn {torn} (first sector stale: {first_half})")
 
 
-# ---- BASELINE configurations at their full sizes ---------------------------
+# ---- the benchmark configurations at their full sizes -----------------------
 def test_config3_broadcast_64mib_8_ranks(dev):
     world, n = 8, 33554432
     root_data = uniform(n, -4.0, 4.0, 2).to(dev)

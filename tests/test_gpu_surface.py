@@ -1,5 +1,6 @@
 """The reference-named operator surface: send / recv / sync, argument checks,
-asynchronous launch, BASELINE config 2 and the allgather sweep of config 5."""
+asynchronous launch, benchmark configuration 2 (256 MiB sendrecv) and the
+allgather sweep of configuration 5."""
 import numpy as np
 import pytest
 import torch

@@ -112,7 +112,7 @@ def test_wrong_flags_are_counted(layout):
 
 @pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
 def test_config1_roundtrip_1mib_fp16(layout):
-    # BASELINE config 1: 524,288 fp16, uniform[-1,1], seed 0; line numbers from
+    # benchmark configuration 1: 524,288 fp16, uniform[-1,1], seed 0; line numbers from
     # 1 (reference) and the constant "step counter 1" variant
     x = uniform(524288, -1.0, 1.0, 0)
     raw = as_bytes(x)
