@@ -13,7 +13,10 @@ import subprocess
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_PKG)
 SO_PATH = os.path.join(_PKG, "libmintccl.so")
-SRC = os.path.join(_PKG, "csrc", "mintccl.hip")
+_CSRC = os.path.join(_PKG, "csrc")
+SRC = os.path.join(_CSRC, "mintccl.hip")
+FAMILY_SRC = os.path.join(_CSRC, "ring_family.hip")     # compiled once per element type
+BUILD_DIR = os.path.join(_PKG, "_build")
 
 MAX_RANKS = 8
 STATUS_WORDS = 4
@@ -27,7 +30,7 @@ OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER, OP_ALLREDU
 PLACE_SPREAD, PLACE_LOCAL = 0, 1
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed FP32 instructions are kept out of all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
@@ -81,13 +84,36 @@ _lib = None
 
 
 def build(verbose: bool = False) -> str:
-    """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree)."""
-    cmd = ["hipcc", *HIPCC_FLAGS, "-o", SO_PATH, SRC]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed:\n{proc.stderr}")
+    """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree).
+
+    The ring kernels are one translation unit per element type; the five
+    compilations run side by side and are linked at the end."""
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    units = [(SRC, [], os.path.join(BUILD_DIR, "mintccl.o"))]
+    for dt in range(4):
+        units.append((FAMILY_SRC, [f"-DMINT_FAMILY_DT={dt}"],
+                      os.path.join(BUILD_DIR, f"ring_family_{dt}.o")))
+    procs = []
+    for src, defs, obj in units:
+        cmd = ["hipcc", *HIPCC_FLAGS, *defs, "-c", "-o", obj, src]
+        if verbose:
+            print(" ".join(cmd))
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                                            text=True)))
+    errors = []
+    for cmd, proc in procs:
+        _, err = proc.communicate()
+        if proc.returncode != 0:
+            errors.append(f"{' '.join(cmd)}\n{err}")
+    if errors:
+        raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
+    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO_PATH,
+            *[obj for _, _, obj in units]]
     if verbose:
-        print(" ".join(cmd))
+        print(" ".join(link))
+    proc = subprocess.run(link, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc link failed:\n{proc.stderr}")
     return SO_PATH
 
 

@@ -6,7 +6,7 @@
 #include <atomic>
 
 #include "kernels.hpp"
-#include "ring.hpp"
+#include "ring_launch.hpp"
 
 using namespace mint;
 
@@ -21,27 +21,11 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
 inline bool aligned16(const void* p) { return aligned16(reinterpret_cast<uint64_t>(p)); }
 
-int device_cus() {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-        return 0;
-    return cus;
-}
-
-int launch_status() { return hipGetLastError() == hipSuccess ? MINT_OK : MINT_ERR_HIP; }
-
 bool reducing(int op) {
     return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE;
 }
 
 // Everything the launch derives from the descriptor.
-struct Plan {
-    RingArgs args;
-    int blocks, threads, unroll;
-    bool empty;
-};
-
 int make_plan(const mint_ring_op* op, Plan* plan) {
     if (!op || !plan) return MINT_ERR_ARG;
     if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLREDUCE) return MINT_ERR_ARG;
@@ -192,51 +176,14 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     return MINT_OK;
 }
 
-template <int PROTO, int DT, int CP>
-int launch_ring_u(const Plan& plan, hipStream_t stream) {
-    void (*kernel)(const RingArgs) = nullptr;
-    switch (plan.unroll) {
-        case 4: kernel = ring_kernel<PROTO, DT, CP, 4>; break;
-        case 2: kernel = ring_kernel<PROTO, DT, CP, 2>; break;
-        default: kernel = ring_kernel<PROTO, DT, CP, 1>; break;
-    }
-    // Every wavefront of the launch polls words other wavefronts write, so
-    // the whole grid has to be resident at once.  The occupancy of a kernel
-    // at a block size does not change: ask once (per block size) and keep it.
-    // (these statics are per template instantiation, i.e. per kernel family)
-    static std::atomic<int> cached[3][9] = {};       // [unroll][threads / 64]
-    static std::atomic<int> cus{0};
-    std::atomic<int>& memo = cached[plan.unroll == 4 ? 2 : (plan.unroll == 2 ? 1 : 0)]
-                                   [plan.threads / 64];
-    int per_cu = memo.load(std::memory_order_relaxed);
-    if (per_cu == 0) {
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) !=
-            hipSuccess)
-            return MINT_ERR_HIP;
-        memo.store(per_cu, std::memory_order_relaxed);
-    }
-    int ncu = cus.load(std::memory_order_relaxed);
-    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
-                       plan.args);
-    return launch_status();
-}
-template <int PROTO, int DT>
-int launch_ring_cp(const Plan& plan, int cache_policy, hipStream_t stream) {
-    switch (cache_policy) {
-        case 0: return launch_ring_u<PROTO, DT, 0>(plan, stream);
-        case 1: return launch_ring_u<PROTO, DT, 1>(plan, stream);
-        default: return launch_ring_u<PROTO, DT, 2>(plan, stream);
-    }
-}
-template <int PROTO>
-int launch_ring_dt(const Plan& plan, int dtype, int cache_policy, hipStream_t stream) {
+// The ring kernels are compiled one element type per translation unit
+// (ring_family.hip), so that the build can run them side by side.
+int launch_ring(const Plan& plan, int protocol, int dtype, int cache_policy, hipStream_t stream) {
     switch (dtype) {
-        case MINT_F16: return launch_ring_cp<PROTO, DT_F16>(plan, cache_policy, stream);
-        case MINT_BF16: return launch_ring_cp<PROTO, DT_BF16>(plan, cache_policy, stream);
-        case MINT_F32: return launch_ring_cp<PROTO, DT_F32>(plan, cache_policy, stream);
-        default: return launch_ring_cp<PROTO, DT_BYTES>(plan, cache_policy, stream);
+        case MINT_F16: return launch_ring_family_f16(plan, protocol, cache_policy, stream);
+        case MINT_BF16: return launch_ring_family_bf16(plan, protocol, cache_policy, stream);
+        case MINT_F32: return launch_ring_family_f32(plan, protocol, cache_policy, stream);
+        default: return launch_ring_family_bytes(plan, protocol, cache_policy, stream);
     }
 }
 
@@ -413,9 +360,7 @@ int mint_ring_launch(const mint_ring_op* op, void* stream) {
     const int err = make_plan(op, &plan);
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
-    return op->protocol == MINT_PROTO_LL128
-               ? launch_ring_dt<PROTO_LL128>(plan, op->dtype, op->cache_policy, as_stream(stream))
-               : launch_ring_dt<PROTO_SIMPLE>(plan, op->dtype, op->cache_policy, as_stream(stream));
+    return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, as_stream(stream));
 }
 
 int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,

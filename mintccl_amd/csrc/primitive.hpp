@@ -73,19 +73,29 @@ __device__ __forceinline__ void st64(const Window& w, uint32_t off, u32x2 v) {
     __builtin_amdgcn_raw_buffer_store_b64(v, w.rsrc, (int)off, 0, CP);
 }
 
+// Pointers into device memory are cast to the global address space before
+// use: a generic pointer makes the compiler emit flat_* instructions, which
+// count on two wait counters at once and so tie vector-memory waits to
+// scalar/LDS ones.
+#define MINT_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ MINT_GLOBAL T* as_global(T* p) {
+    return (MINT_GLOBAL T*)p;
+}
+
 // 64-bit words shared between workgroups (credits, status): relaxed atomics
 // at agent scope compile to global_load/store_dwordx2 ... sc1.
 __device__ __forceinline__ uint64_t ld64_agent(const uint64_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st64_agent(uint64_t* p, uint64_t v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // Plain 64-bit store (no scope bits): stays in the L2 of the XCD that runs the
 // wave.  Relaxed atomic at wavefront scope, so the compiler keeps it whole and
 // in program order with respect to other atomics.
 __device__ __forceinline__ void st64_local(uint64_t* p, uint64_t v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
 // Release for data that was stored with scope bits (write-through) or, for the
 // XCD-local policy, into the L2 both sides share: once the wave's stores are
@@ -99,16 +109,16 @@ __device__ __forceinline__ void wait_stores_visible() {
 
 // Streaming accesses to the caller's buffers (read once / written once).
 __device__ __forceinline__ u32x4 ld128_stream(const void* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x4*>(p)));
 }
 __device__ __forceinline__ void st128_stream(void* p, u32x4 v) {
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+    __builtin_nontemporal_store(v, as_global(reinterpret_cast<u32x4*>(p)));
 }
 __device__ __forceinline__ u32x2 ld64_stream(const void* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    return __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2*>(p)));
 }
 __device__ __forceinline__ void st64_stream(void* p, u32x2 v) {
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+    __builtin_nontemporal_store(v, as_global(reinterpret_cast<u32x2*>(p)));
 }
 
 // ---- element addition: one IEEE round-to-nearest-even per call ------------

@@ -52,18 +52,19 @@ struct LaneMap {
 
 // Byte-granular guarded access for the ragged end of a buffer: reads
 // [off, off + len) clipped to nbytes, missing bytes read as zero.
-__device__ __forceinline__ u32x4 load_guarded(const uint8_t* base, uint64_t off, uint32_t len,
+__device__ __forceinline__ u32x4 load_guarded(const uint8_t* base_, uint64_t off, uint32_t len,
                                               uint64_t nbytes) {
+    MINT_GLOBAL const uint8_t* base = as_global(base_);
     u32x4 v = {0u, 0u, 0u, 0u};
     if (off >= nbytes) return v;
     uint64_t have = nbytes - off;
     if (have >= len) {
-        if (len == 16u) return *reinterpret_cast<const u32x4*>(base + off);
+        if (len == 16u) return *(MINT_GLOBAL const u32x4*)(base + off);
         if (len == 12u) {
-            u32x3 h = *reinterpret_cast<const u32x3_a4*>(base + off);
+            u32x3 h = *(MINT_GLOBAL const u32x3_a4*)(base + off);
             v.x = h.x; v.y = h.y; v.z = h.z;
         } else {                                   // 8
-            u32x2 h = *reinterpret_cast<const u32x2*>(base + off);
+            u32x2 h = *(MINT_GLOBAL const u32x2*)(base + off);
             v.x = h.x; v.y = h.y;
         }
         return v;
@@ -74,18 +75,19 @@ __device__ __forceinline__ u32x4 load_guarded(const uint8_t* base, uint64_t off,
     v.x = w[0]; v.y = w[1]; v.z = w[2]; v.w = w[3];
     return v;
 }
-__device__ __forceinline__ void store_guarded(uint8_t* base, uint64_t off, uint32_t len,
+__device__ __forceinline__ void store_guarded(uint8_t* base_, uint64_t off, uint32_t len,
                                               uint64_t nbytes, u32x4 v) {
+    MINT_GLOBAL uint8_t* base = as_global(base_);
     if (off >= nbytes) return;
     uint64_t have = nbytes - off;
     if (have >= len) {
-        if (len == 16u) { *reinterpret_cast<u32x4*>(base + off) = v; return; }
+        if (len == 16u) { *(MINT_GLOBAL u32x4*)(base + off) = v; return; }
         if (len == 12u) {
             u32x3 h = {v.x, v.y, v.z};
-            *reinterpret_cast<u32x3_a4*>(base + off) = h;
+            *(MINT_GLOBAL u32x3_a4*)(base + off) = h;
         } else {                                   // 8
             u32x2 h = {v.x, v.y};
-            *reinterpret_cast<u32x2*>(base + off) = h;
+            *(MINT_GLOBAL u32x2*)(base + off) = h;
         }
         return;
     }
@@ -95,68 +97,53 @@ __device__ __forceinline__ void store_guarded(uint8_t* base, uint64_t off, uint3
 }
 
 // ---- wave64 LL128 block: raw side ----------------------------------------
-// load_ll128 (protocol.py:57-85): raw block g of a row -> registers.  On
-// flag lanes .x/.y/.z hold the 12 payload bytes; .w is don't-care.
-__device__ __forceinline__ u32x4 ll_load_raw(const uint8_t* row, uint64_t row_bytes, uint32_t g,
-                                             const LaneMap& m) {
+// load_ll128 (protocol.py:57-85) in two halves, so that the load can be in
+// flight while the wave does something else: ll_fetch_raw issues the load of
+// raw block g of a row, ll_arrange (to be called where the value is first
+// needed) puts the 12 payload bytes of a flag lane into .x/.y/.z; .w is
+// don't-care there.  `full` (wave-uniform) says the block lies wholly inside
+// the row; the ragged last block is read byte-guarded and arrives arranged.
+__device__ __forceinline__ u32x4 ll_fetch_raw(const uint8_t* row, uint64_t row_bytes, uint32_t g,
+                                              bool full, const LaneMap& m) {
     const uint64_t base = (uint64_t)g * kBlockRawLL;
-    u32x4 v;
-    if (base + kBlockRawLL <= row_bytes) {       // wave-uniform
+    if (full) {
         // flag lanes start 4 bytes early so that all 64 lanes issue one
         // 16-byte load that stays inside the block
         const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
-        v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a4*>(row + base + off));
-        if (m.flag_lane) { v.x = v.y; v.y = v.z; v.z = v.w; }
-    } else {
-        v = load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
+        return __builtin_nontemporal_load(
+            (MINT_GLOBAL const u32x4_a4*)(row + base + off));
     }
+    return load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
+}
+__device__ __forceinline__ u32x4 ll_arrange(u32x4 v, bool full, const LaneMap& m) {
+    if (full && m.flag_lane) { v.x = v.y; v.y = v.z; v.z = v.w; }
     return v;
 }
-// The same through a buffer window, with an explicit cache policy (rows of
-// less than 4 GiB; the ragged last block still goes through the pointer).
-template <int CP>
-__device__ __forceinline__ u32x4 ll_load_raw_w(const Window& win, const uint8_t* row,
-                                               uint64_t row_bytes, uint32_t g, const LaneMap& m) {
-    const uint64_t base = (uint64_t)g * kBlockRawLL;
-    u32x4 v;
-    if (base + kBlockRawLL <= row_bytes) {
-        const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
-        v = ld128<CP>(win, (uint32_t)base + off);
-        if (m.flag_lane) { v.x = v.y; v.y = v.z; v.z = v.w; }
-    } else {
-        v = load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
-    }
-    return v;
-}
-template <int CP>
-__device__ __forceinline__ void ll_save_raw_w(const Window& win, uint8_t* row, uint64_t row_bytes,
-                                              uint32_t g, const LaneMap& m, u32x4 v) {
-    const uint64_t base = (uint64_t)g * kBlockRawLL;
-    if (base + kBlockRawLL <= row_bytes) {
-        if (!m.flag_lane) {
-            st128<CP>(win, (uint32_t)base + m.raw_off, v);
-        } else {
-            u32x3 h = {v.x, v.y, v.z};
-            __builtin_amdgcn_raw_buffer_store_b96(h, win.rsrc, (int)((uint32_t)base + m.raw_off), 0, CP);
-        }
-    } else {
-        store_guarded(row, base + m.raw_off, m.raw_len, row_bytes, v);
-    }
+__device__ __forceinline__ u32x4 ll_load_raw(const uint8_t* row, uint64_t row_bytes, uint32_t g,
+                                             const LaneMap& m) {
+    const bool full = (uint64_t)g * kBlockRawLL + kBlockRawLL <= row_bytes;    // wave-uniform
+    return ll_arrange(ll_fetch_raw(row, row_bytes, g, full, m), full, m);
 }
 // save_ll128 (protocol.py:87-100): registers -> raw block g of a row.
-__device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, uint32_t g,
+__device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, uint32_t g, bool full,
                                             const LaneMap& m, u32x4 v) {
     const uint64_t base = (uint64_t)g * kBlockRawLL;
-    if (base + kBlockRawLL <= row_bytes) {
+    if (full) {
         if (!m.flag_lane) {
             st128_stream(row + base + m.raw_off, v);
         } else {
             u32x3 h = {v.x, v.y, v.z};
-            __builtin_nontemporal_store(h, reinterpret_cast<u32x3_a4*>(row + base + m.raw_off));
+            __builtin_nontemporal_store(
+                h, (MINT_GLOBAL u32x3_a4*)(row + base + m.raw_off));
         }
     } else {
         store_guarded(row, base + m.raw_off, m.raw_len, row_bytes, v);
     }
+}
+__device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, uint32_t g,
+                                            const LaneMap& m, u32x4 v) {
+    const bool full = (uint64_t)g * kBlockRawLL + kBlockRawLL <= row_bytes;    // wave-uniform
+    ll_save_raw(row, row_bytes, g, full, m, v);
 }
 
 // ---- wave64 LL128 block: message side ------------------------------------

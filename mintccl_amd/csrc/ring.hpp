@@ -33,6 +33,8 @@
 // reuses a slot - separate from the data lines, unlike wait/post_ll128 which
 // overload the flag word of slot 0.
 #pragma once
+#include <type_traits>
+
 #include "protocol.hpp"
 
 namespace mint {
@@ -160,9 +162,294 @@ template <> struct Policy<0> { static constexpr int LD = CP_SC1, ST = CP_SC1; };
 template <> struct Policy<1> { static constexpr int LD = CP_SYSTEM, ST = CP_SYSTEM; };
 template <> struct Policy<2> { static constexpr int LD = CP_SC1, ST = CP_NONE; };
 
+// A role whose flags are compile-time constants.
+template <bool LOAD, bool RECV, bool REDUCE, bool SAVE, bool SEND>
+struct FixedRole {
+    int rank, next;
+    static constexpr bool load = LOAD, recv = RECV, reduce = REDUCE, save = SAVE, send = SEND;
+};
+
+// The walk of one wave-channel along its rows, specialised by what its
+// position does (the flags are compile-time constants so that the loop of an
+// origin, an adder, a copier or a sink carries no tests for the other roles).
+template <int PROTO, int DT, int CPI, int U, typename RoleT>
+__device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const int h, const int w,
+                                          const RoleT role) {
+    constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
+    const LaneMap m;
+    const uint64_t row_off = (uint64_t)p * a.row_stride;
+    // allreduce splits one buffer into `world` rows; the last ones may be short or empty
+    uint64_t row_bytes = a.row_bytes;
+    uint32_t nblocks = a.nblocks;
+    if (a.total_bytes) {
+        const uint64_t left = a.total_bytes > row_off ? a.total_bytes - row_off : 0;
+        row_bytes = left < a.row_bytes ? left : a.row_bytes;
+        const uint32_t per_block = PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
+        nblocks = (uint32_t)((row_bytes + per_block - 1) / per_block);
+    }
+    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
+    uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
+    // blocks that lie wholly inside the row take the unguarded path
+    const uint32_t nfull = (uint32_t)(row_bytes / (PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple));
+    const uint32_t ring_bytes = a.nslots * a.slot_bytes;
+    const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
+    const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);
+    // a rank can receive twice in one pipeline of an allreduce (once while
+    // the sum is built, once while it is handed round): each phase has its own
+    // share of the slots and its own credit words
+    const uint32_t share_recv = (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
+    const uint32_t share_send = (uint32_t)p * (uint32_t)a.phases + (h + 1 >= a.world && a.phases > 1 ? 1u : 0u);
+    const uint32_t own_chan = a.credit_off + (share_recv * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
+    const uint32_t nxt_chan = a.credit_off + (share_send * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
+    uint64_t* own_tail = reinterpret_cast<uint64_t*>(a.staging[role.rank] + own_chan);
+    uint64_t* own_head = own_tail + 16;
+    uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + nxt_chan);
+    uint64_t* nxt_head = nxt_tail + 16;
+
+    const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
+    const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
+    const uint32_t groups_per_step = K / U;
+    const uint32_t ngroups = a.steps * groups_per_step;
+    uint32_t credits_seen = 0, head_seen = 0;
+    // wait accounting, 10 ns ticks: only in a library built with
+    // -DMINT_RING_STATS (it costs scalar registers, hence occupancy)
+#ifdef MINT_RING_STATS
+    const bool timing = a.stats != nullptr;
+#else
+    constexpr bool timing = false;
+#endif
+    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
+    const uint64_t t_begin = timing ? wall_clock64() : 0;
+
+    // Group = U blocks of this wave-channel inside one step.  The walk over
+    // (step, first block) is kept incrementally: no division in the loop.
+    struct Group { uint32_t step, slot, k0, idx[U], g[U]; bool valid[U], full[U], first, last; };
+    auto fill = [&](Group& q) {
+        q.first = q.k0 == 0;
+        q.last = q.k0 + (uint32_t)U >= K;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            q.idx[u] = (q.k0 + (uint32_t)u) * W + (uint32_t)w;
+            q.g[u] = q.step * a.step_blocks + q.idx[u];
+            q.valid[u] = q.g[u] < nblocks;
+            q.full[u] = q.g[u] < nfull;
+        }
+    };
+    auto first_group = [&]() {
+        Group q;
+        q.step = 0; q.slot = 0; q.k0 = 0;
+        fill(q);
+        return q;
+    };
+    auto next_group = [&](const Group& cur) {
+        Group q;
+        q.step = cur.step; q.slot = cur.slot; q.k0 = cur.k0 + (uint32_t)U;
+        if (q.k0 >= K) {
+            q.k0 = 0;
+            ++q.step;
+            q.slot = cur.slot + 1 == a.nslots ? 0 : cur.slot + 1;
+        }
+        fill(q);
+        return q;
+    };
+    // load_ll128 of the wave's own rows for one group: only the loads;
+    // arrange_own finishes the job where the values are needed.
+    auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            v[u] = u32x4{0u, 0u, 0u, 0u};
+            if (!q.valid[u]) continue;
+            if (PROTO == PROTO_LL128) {
+                v[u] = ll_fetch_raw(in_row, row_bytes, q.g[u], q.full[u], m);
+            } else {
+                const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
+                v[u] = q.full[u] ? ld128_stream(in_row + off)
+                                 : load_guarded(in_row, off, 16u, row_bytes);
+            }
+        }
+    };
+    // The same for a group that may lie beyond the part of the row made of
+    // whole blocks: block numbers are clamped to the last whole block, so the
+    // loads are issued unconditionally and always land inside the row (what
+    // they bring is only used if the group turns out to be a whole one).
+    // Needs nfull >= 1.
+    auto fetch_ahead = [&](const Group& q, u32x4 (&v)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t g = q.g[u] < nfull ? q.g[u] : nfull - 1u;
+            if (PROTO == PROTO_LL128)
+                v[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
+            else
+                v[u] = ld128_stream(in_row + (uint64_t)g * kBlockRawSimple + m.lane * 16u);
+        }
+    };
+
+    u32x4 v[U], vnext[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
+    Group q = first_group();
+    uint32_t n = 0;
+    // Loop-carried, and looked at in every iteration whether or not a credit
+    // was asked for: the compiler then knows that no load into these
+    // registers is outstanding at the top of the loop and does not have to
+    // drain the memory pipeline (and with it the fetch-ahead) there.
+    uint64_t credit_word = 0;
+
+    // One group.  WHOLE = every block of the group lies wholly inside the row:
+    // then nothing in the body depends on per-block validity, the own rows of
+    // the following group are fetched ahead, and - what the arrangement is
+    // for - the number of loads issued after the first polls is the same on
+    // every path, so the wait for the polls leaves exactly the fetch-ahead in
+    // flight: it has a whole group's time to come back from HBM.  The other
+    // groups (the ragged end of a row, a step that is only partly filled) take
+    // the guarded body and load their own rows on the spot.
+    auto run_group = [&](auto whole_tag) -> bool {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
+        const Group qn = next_group(q);
+        const uint32_t s = q.step;
+        const uint32_t slot_off = q.slot * a.slot_bytes + share_recv * a.step_msg;
+        const uint32_t send_off = q.slot * a.slot_bytes + share_send * a.step_msg;
+        const uint32_t tag = (a.epoch << 20) | (s + 1u);
+        // wait_ll128 (protocol.py:161-180): the credit for the slot this step
+        // goes into is only needed before the send, so its load is issued
+        // here, ahead of the polls, and looked at after them.
+        const uint32_t need = s >= a.nslots ? s - a.nslots + 1 : 0;
+        const bool ask_credit = q.first && role.send && credits_seen < need;
+        if (ask_credit) credit_word = ld64_agent(nxt_tail);
+        if (q.first && PROTO == PROTO_SIMPLE && role.recv) {
+            const uint64_t t0 = timing ? wall_clock64() : 0;
+            if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status)) {
+                report_timeout(a.status, p, h, w, s);
+                return false;
+            }
+            if (timing) t_credit += wall_clock64() - t0;
+        }
+        u32x4 r[U];
+        const uint64_t t1 = timing ? wall_clock64() : 0;
+        if (role.recv) {
+            // first poll of recv_ll128 (protocol.py:102-130): loads only
+            compiler_fence();
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (WHOLE || q.valid[u])
+                    r[u] = ld128<LDCP>(own, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u);
+        }
+        if (role.load) {
+            if (WHOLE) fetch_ahead(qn, vnext);
+            else load_own(q, v);
+        }
+        if (role.recv && PROTO == PROTO_LL128) {
+            uint32_t pending = 0;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if ((WHOLE || q.valid[u]) && !wave_all(!m.flag_lane || r[u].w == tag))
+                    pending |= 1u << u;
+            for (uint32_t spins = 0; pending; ++spins) {
+                if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
+                    report_timeout(a.status, p, h, w, s);
+                    return false;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                compiler_fence();
+                ++n_repoll;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (!(pending & (1u << u))) continue;
+                    if (ll_poll<LDCP>(own, slot_off + q.idx[u] * kBlockMsg, tag, m, r[u]))
+                        pending &= ~(1u << u);
+                }
+            }
+        }
+        if (timing) { t_poll += wall_clock64() - t1; ++n_groups; }
+        asm volatile("" : "+v"(credit_word));
+        if (ask_credit) {
+            const uint64_t t0 = timing ? wall_clock64() : 0;
+            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(credit_word >> 32));
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)credit_word);
+            if (hi == a.epoch && lo >= need) {
+                credits_seen = lo;
+            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
+                                   a.status)) {
+                report_timeout(a.status, p, h, w, s);
+                return false;
+            }
+            if (timing) t_credit += wall_clock64() - t0;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!(WHOLE || q.valid[u])) continue;
+            const bool full = WHOLE || q.full[u];
+            if (role.load && PROTO == PROTO_LL128) v[u] = ll_arrange(v[u], full, m);
+            if (role.recv) {
+                if constexpr (DT != DT_BYTES) {
+                    v[u] = role.reduce ? ll_comp<DT>(v[u], r[u]) : r[u];
+                } else {
+                    v[u] = r[u];
+                }
+            }
+            if (role.save) {
+                if (PROTO == PROTO_LL128) {
+                    ll_save_raw(out_row, row_bytes, q.g[u], full, m, v[u]);
+                } else {
+                    const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
+                    if (full) st128_stream(out_row + off, v[u]);
+                    else store_guarded(out_row, off, 16u, row_bytes, v[u]);
+                }
+            }
+            if (role.send) {
+                if (PROTO == PROTO_LL128)
+                    ll_send<STCP>(nxt, send_off + q.idx[u] * kBlockMsg, v[u], tag, m);
+                else
+                    st128<STCP>(nxt, send_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
+            }
+        }
+        if (q.last) {
+            // post_ll128 (protocol.py:183-189): this wave-channel has taken every
+            // line of step s out of its slot (the loads have returned: their
+            // values were tested / used above).
+            if (role.recv && lane_id() == 0) {
+                if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
+                else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
+            }
+            if (PROTO == PROTO_SIMPLE && role.send) {
+                // Simple protocol: data first, then the step counter.  The data
+                // loads of the receiver skip the L1 (LDCP), so no invalidate.
+                wait_stores_visible();
+                if (lane_id() == 0) {
+                    if (STCP == CP_NONE) st64_local(nxt_head, flag_hi | (uint64_t)(s + 1));
+                    else st64_agent(nxt_head, flag_hi | (uint64_t)(s + 1));
+                }
+            }
+        }
+        if (WHOLE) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = vnext[u];
+        }
+        q = qn;
+        ++n;
+        return true;
+    };
+
+    // block numbers grow from group to group, so the whole groups come first
+    if (role.load && ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
+    while (n < ngroups && q.g[U - 1] < nfull)
+        if (!run_group(std::true_type{})) return;
+    while (n < ngroups)
+        if (!run_group(std::false_type{})) return;
+
+    if (timing && lane_id() == 0) {
+        unsigned long long* st = reinterpret_cast<unsigned long long*>(a.stats) + 8 * h;
+        atomicAdd(st + 0, (unsigned long long)n_groups);
+        atomicAdd(st + 1, (unsigned long long)n_repoll);
+        atomicAdd(st + 2, (unsigned long long)t_credit);
+        atomicAdd(st + 3, (unsigned long long)t_poll);
+        atomicAdd(st + 4, (unsigned long long)(wall_clock64() - t_begin));
+        atomicAdd(st + 5, 1ull);
+    }
+}
+
 template <int PROTO, int DT, int CPI, int U>
 __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
-    constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
     const int npos = a.hops + 1;
     const int x = (int)blockIdx.x;
     int c, h;
@@ -203,240 +490,29 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const Role role = role_of(a, p, h);
     if (h == 0 && a.skip_origin) return;
 
-    const LaneMap m;
-    const uint64_t row_off = (uint64_t)p * a.row_stride;
-    // allreduce splits one buffer into `world` rows; the last ones may be short or empty
-    uint64_t row_bytes = a.row_bytes;
-    uint32_t nblocks = a.nblocks;
-    if (a.total_bytes) {
-        const uint64_t left = a.total_bytes > row_off ? a.total_bytes - row_off : 0;
-        row_bytes = left < a.row_bytes ? left : a.row_bytes;
-        const uint32_t per_block = PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
-        nblocks = (uint32_t)((row_bytes + per_block - 1) / per_block);
-    }
-    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
-    uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
-#if defined(MINT_RAW_LD_CP) || defined(MINT_RAW_ST_CP)
-    const Window in_w(in_row, (uint32_t)row_bytes), out_w(out_row, (uint32_t)row_bytes);
-#endif
-    const uint32_t ring_bytes = a.nslots * a.slot_bytes;
-    const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
-    const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);
-    // a rank can receive twice in one pipeline of an allreduce (once while
-    // the sum is built, once while it is handed round): each phase has its own
-    // share of the slots and its own credit words
-    const uint32_t share_recv = (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
-    const uint32_t share_send = (uint32_t)p * (uint32_t)a.phases + (h + 1 >= a.world && a.phases > 1 ? 1u : 0u);
-    const uint32_t own_chan = a.credit_off + (share_recv * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
-    const uint32_t nxt_chan = a.credit_off + (share_send * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
-    uint64_t* own_tail = reinterpret_cast<uint64_t*>(a.staging[role.rank] + own_chan);
-    uint64_t* own_head = own_tail + 16;
-    uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + nxt_chan);
-    uint64_t* nxt_head = nxt_tail + 16;
-
-    const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
-    const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
-    const uint32_t groups_per_step = K / U;
-    const uint32_t ngroups = a.steps * groups_per_step;
-    uint32_t credits_seen = 0, head_seen = 0;
-    // wait accounting, 10 ns ticks: only in a library built with
-    // -DMINT_RING_STATS (it costs scalar registers, hence occupancy)
-#ifdef MINT_RING_STATS
-    const bool timing = a.stats != nullptr;
+#ifdef MINT_RING_GENERIC_ROLE
+    ring_walk<PROTO, DT, CPI, U>(a, p, h, w, role);
 #else
-    constexpr bool timing = false;
-#endif
-    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
-    const uint64_t t_begin = timing ? wall_clock64() : 0;
-
-    // Group = U blocks of this wave-channel inside one step.  The walk over
-    // (step, first block) is kept incrementally: no division in the loop.
-    struct Group { uint32_t step, slot, k0, idx[U], g[U]; bool valid[U], first, last; };
-    auto fill = [&](Group& q) {
-        q.first = q.k0 == 0;
-        q.last = q.k0 + (uint32_t)U >= K;
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            q.idx[u] = (q.k0 + (uint32_t)u) * W + (uint32_t)w;
-            q.g[u] = q.step * a.step_blocks + q.idx[u];
-            q.valid[u] = q.g[u] < nblocks;
+    // one specialised walk per role
+    const int rk = role.rank, nx = role.next;
+    if (!role.recv) {
+        ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, false, false, false, true>{rk, nx});
+    } else if (role.reduce) {
+        if constexpr (DT != DT_BYTES) {
+            if (role.save)
+                ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, true, true, true, true>{rk, nx});
+            else
+                ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, true, true, false, true>{rk, nx});
         }
-    };
-    auto first_group = [&]() {
-        Group q;
-        q.step = 0; q.slot = 0; q.k0 = 0;
-        fill(q);
-        return q;
-    };
-    auto next_group = [&](const Group& cur) {
-        Group q;
-        q.step = cur.step; q.slot = cur.slot; q.k0 = cur.k0 + (uint32_t)U;
-        if (q.k0 >= K) {
-            q.k0 = 0;
-            ++q.step;
-            q.slot = cur.slot + 1 == a.nslots ? 0 : cur.slot + 1;
-        }
-        fill(q);
-        return q;
-    };
-    // load_ll128 of the wave's own rows for one group.
-    auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            v[u] = u32x4{0u, 0u, 0u, 0u};
-            if (!q.valid[u]) continue;
-            if (PROTO == PROTO_LL128) {
-#ifdef MINT_RAW_LD_CP
-                v[u] = ll_load_raw_w<MINT_RAW_LD_CP>(in_w, in_row, row_bytes, q.g[u], m);
-#else
-                v[u] = ll_load_raw(in_row, row_bytes, q.g[u], m);
-#endif
-            } else {
-                const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                v[u] = off + 16u <= row_bytes ? ld128_stream(in_row + off)
-                                               : load_guarded(in_row, off, 16u, row_bytes);
-            }
-        }
-    };
-
-    // The own rows do not depend on anybody, so they are fetched one group
-    // ahead: the load for group n + 1 is issued right after the first poll of
-    // group n (younger than the poll, so waiting for the poll does not wait
-    // for it) and has a whole group's time to come back from HBM.
-    u32x4 v[U], vnext[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
-    Group q = first_group();
-    if (role.load && ngroups) load_own(q, v);
-
-    for (uint32_t n = 0; n < ngroups; ++n) {
-        const Group qn = next_group(q);
-        const uint32_t s = q.step;
-        const uint32_t slot_off = q.slot * a.slot_bytes + share_recv * a.step_msg;
-        const uint32_t send_off = q.slot * a.slot_bytes + share_send * a.step_msg;
-        const uint32_t tag = (a.epoch << 20) | (s + 1u);
-        // wait_ll128 (protocol.py:161-180): the credit for the slot this step
-        // goes into is only needed before the send, so its load is issued
-        // here, ahead of the polls, and looked at after them.
-        const uint32_t need = s >= a.nslots ? s - a.nslots + 1 : 0;
-        const bool ask_credit = q.first && role.send && credits_seen < need;
-        uint64_t credit_word = 0;
-        if (ask_credit) credit_word = ld64_agent(nxt_tail);
-        if (q.first && PROTO == PROTO_SIMPLE && role.recv) {
-            const uint64_t t0 = timing ? wall_clock64() : 0;
-            if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status)) {
-                report_timeout(a.status, p, h, w, s);
-                return;
-            }
-            if (timing) t_credit += wall_clock64() - t0;
-        }
-        u32x4 r[U];
-        const uint64_t t1 = timing ? wall_clock64() : 0;
-        if (role.recv) {
-            // first poll of recv_ll128 (protocol.py:102-130): loads only
-            compiler_fence();
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (q.valid[u])
-                    r[u] = ld128<LDCP>(own, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u);
-        }
-        if (role.load && n + 1 < ngroups) load_own(qn, vnext);
-        if (role.recv && PROTO == PROTO_LL128) {
-            uint32_t pending = 0;
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (q.valid[u] && !wave_all(!m.flag_lane || r[u].w == tag)) pending |= 1u << u;
-            for (uint32_t spins = 0; pending; ++spins) {
-                if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
-                    report_timeout(a.status, p, h, w, s);
-                    return;
-                }
-                __builtin_amdgcn_s_sleep(1);
-                compiler_fence();
-                ++n_repoll;
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (!(pending & (1u << u))) continue;
-                    if (ll_poll<LDCP>(own, slot_off + q.idx[u] * kBlockMsg, tag, m, r[u]))
-                        pending &= ~(1u << u);
-                }
-            }
-        }
-        if (timing) { t_poll += wall_clock64() - t1; ++n_groups; }
-        if (ask_credit) {
-            const uint64_t t0 = timing ? wall_clock64() : 0;
-            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(credit_word >> 32));
-            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)credit_word);
-            if (hi == a.epoch && lo >= need) {
-                credits_seen = lo;
-            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
-                                   a.status)) {
-                report_timeout(a.status, p, h, w, s);
-                return;
-            }
-            if (timing) t_credit += wall_clock64() - t0;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (!q.valid[u]) continue;
-            if (role.recv) {
-                if constexpr (DT != DT_BYTES) {
-                    v[u] = role.reduce ? ll_comp<DT>(v[u], r[u]) : r[u];
-                } else {
-                    v[u] = r[u];
-                }
-            }
-            if (role.save) {
-                if (PROTO == PROTO_LL128) {
-#ifdef MINT_RAW_ST_CP
-                    ll_save_raw_w<MINT_RAW_ST_CP>(out_w, out_row, row_bytes, q.g[u], m, v[u]);
-#else
-                    ll_save_raw(out_row, row_bytes, q.g[u], m, v[u]);
-#endif
-                } else {
-                    const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                    if (off + 16u <= row_bytes) st128_stream(out_row + off, v[u]);
-                    else store_guarded(out_row, off, 16u, row_bytes, v[u]);
-                }
-            }
-            if (role.send) {
-                if (PROTO == PROTO_LL128)
-                    ll_send<STCP>(nxt, send_off + q.idx[u] * kBlockMsg, v[u], tag, m);
-                else
-                    st128<STCP>(nxt, send_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
-            }
-        }
-        if (q.last) {
-            // post_ll128 (protocol.py:183-189): this wave-channel has taken every
-            // line of step s out of its slot (the loads have returned: their
-            // values were tested / used above).
-            if (role.recv && lane_id() == 0) {
-                if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
-                else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
-            }
-            if (PROTO == PROTO_SIMPLE && role.send) {
-                // Simple protocol: data first, then the step counter.  The data
-                // loads of the receiver skip the L1 (LDCP), so no invalidate.
-                wait_stores_visible();
-                if (lane_id() == 0) {
-                    if (STCP == CP_NONE) st64_local(nxt_head, flag_hi | (uint64_t)(s + 1));
-                    else st64_agent(nxt_head, flag_hi | (uint64_t)(s + 1));
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = vnext[u];
-        q = qn;
+    } else if (role.send) {
+        if (role.save)
+            ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<false, true, false, true, true>{rk, nx});
+        else
+            ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<false, true, false, false, true>{rk, nx});
+    } else {
+        ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<false, true, false, true, false>{rk, nx});
     }
-    if (timing && lane_id() == 0) {
-        unsigned long long* st = reinterpret_cast<unsigned long long*>(a.stats) + 8 * h;
-        atomicAdd(st + 0, (unsigned long long)n_groups);
-        atomicAdd(st + 1, (unsigned long long)n_repoll);
-        atomicAdd(st + 2, (unsigned long long)t_credit);
-        atomicAdd(st + 3, (unsigned long long)t_poll);
-        atomicAdd(st + 4, (unsigned long long)(wall_clock64() - t_begin));
-        atomicAdd(st + 5, 1ull);
-    }
+#endif
 }
 
 }  // namespace mint
