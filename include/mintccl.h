@@ -135,6 +135,14 @@ int mint_xcd_map(int blocks, void* out, void* stream);
 int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int threads,
                      void* stream);
 
+/* Read-only pass over a buffer: XORs every whole 16-byte vector of
+ * src[0, nbytes) into out (device uint32[4], which the caller has zeroed; the
+ * kernel only XORs into it).  No counterpart in the reference: it is the HBM
+ * read-bandwidth yardstick beside mint_copy_simple, and its result can be
+ * checked.  blocks = 0 picks a device-filling grid. */
+int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int threads,
+                  void* stream);
+
 /* Standalone LL128 codec (load_ll128 + send_ll128 / recv_ll128 + save_ll128,
  * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride:
  * MINT_LAYOUT_PAIR is the reference's wire format (120 payload bytes, then the

@@ -9,6 +9,7 @@ on one GPU they reduce to a device choice and a pointer mailbox.
 from __future__ import annotations
 
 import contextlib
+import math
 import os
 import threading
 import time
@@ -103,10 +104,20 @@ class Timer:
         print(f"# {tag}time: {self.elapsed}s")
 
 
-# Tuned geometry for MI355X (measured): about 4600 wavefronts in flight in
-# total, one 1 KiB block per wave-channel per step, 3 slots; a slot may grow to
-# this many bytes when a collective has few pipelines and hops.
+# Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
+# step.  Collectives with one pipeline per rank (allgather, reducescatter,
+# allreduce): 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in all
+# (from about 6100 on the grid no longer runs as one wave of blocks and the
+# time jumps by a third).  Collectives with a single pipeline (sendrecv,
+# broadcast, reduce): 3 slots of 512 KiB, 4608 wavefronts; a slot may grow to
+# TUNED_SLOT_BUDGET bytes when there are few hops.  Staging is allocated for
+# TUNED_NSLOTS slots of TUNED_SLOT_BUDGET either way.
 TUNED_TOTAL_WAVES = 4608
+TUNED_SLOT_BLOCKS = 512
+TUNED_NSLOTS = 3
+TUNED_TOTAL_WAVES_MULTI = 5760
+TUNED_SLOT_BLOCKS_MULTI = 640
+TUNED_NSLOTS_MULTI = 2
 TUNED_SLOT_BUDGET = 2304 * 1024
 
 
@@ -159,7 +170,7 @@ class VirtualComm:
         self.auto_geometry = (tuned and buff_size_ is None and nslots is None
                               and waves_per_rank is None)
         if nslots is None:
-            nslots = num_slots() if (reference_geometry or buff_size_ is not None) else 3
+            nslots = num_slots() if (reference_geometry or buff_size_ is not None) else TUNED_NSLOTS
         if buff_size_ is None:
             buff_size_ = buff_size() if reference_geometry else nslots * TUNED_SLOT_BUDGET
         self.buff_size, self.nslots = buff_size_, nslots
@@ -282,12 +293,20 @@ class VirtualComm:
             receivers = max(1, min(npos - 1, self.world_size))
             if op == _lib.OP_ALLREDUCE:
                 npos = (npos + 1) // 2        # `pipes` already counts both phases
-            # a slot of 512 KiB per 8 receiving ranks keeps the staging of an
-            # XCD's channels (3 slots x receivers / 8) inside its L2
-            slot_blocks = min(512 * max(1, 8 // receivers), TUNED_TOTAL_WAVES // npos,
+            # slots sized per 8 receiving ranks keep the staging of an XCD's
+            # channels (slots x receivers / 8) well inside its 4 MiB of L2
+            multi = pipes > 1
+            per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
+            total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
+            nslots = min(self.nslots, TUNED_NSLOTS_MULTI) if multi else self.nslots
+            slot_blocks = min(per8 * max(1, 8 // receivers), total // npos,
                               TUNED_SLOT_BUDGET // 1024)
-            waves = max(32, slot_blocks // pipes // 32 * 32)
-            d.slot_bytes, d.nslots = pipes * waves * 1024, self.nslots
+            # whole thread blocks, and a channel count the 8 XCDs divide
+            real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
+            wpb = max(1, self.threads_per_block // 64)
+            granule = wpb * (8 // math.gcd(real_pipes, 8))
+            waves = max(granule, slot_blocks // pipes // granule * granule)
+            d.slot_bytes, d.nslots = pipes * waves * 1024, nslots
             d.waves_per_channel_group = waves
         else:
             d.slot_bytes, d.nslots = self.slot_bytes, self.nslots

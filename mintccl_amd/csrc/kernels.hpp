@@ -5,16 +5,20 @@
 
 namespace mint {
 
-// recv_kernel (1_sendrecv_direct.py:31-54): persistent grid-stride copy,
-// 16 bytes per lane, four independent accesses in flight per lane.
+// recv_kernel (1_sendrecv_direct.py:31-54): persistent copy, 16 bytes per
+// lane, four independent accesses in flight per lane.  Every block walks a
+// contiguous share of the buffer (measured: a grid-stride walk loses up to a
+// fifth of the HBM bandwidth once the grid exceeds one block per CU).
 __global__ void __launch_bounds__(1024) copy_simple_kernel(const uint8_t* __restrict__ src,
                                                            uint8_t* __restrict__ dst,
                                                            uint64_t nbytes) {
     const uint64_t nvec = nbytes >> 4;
-    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
-    uint64_t i = tid;
-    for (; i + 3 * nthr < nvec; i += 4 * nthr) {
+    const uint64_t per = (nvec + gridDim.x - 1) / gridDim.x;
+    const uint64_t lo = (uint64_t)blockIdx.x * per;
+    const uint64_t hi = lo + per < nvec ? lo + per : nvec;
+    const uint64_t nthr = blockDim.x;
+    uint64_t i = lo + threadIdx.x;
+    for (; i + 3 * nthr < hi; i += 4 * nthr) {
         u32x4 a = ld128_stream(src + (i << 4));
         u32x4 b = ld128_stream(src + ((i + nthr) << 4));
         u32x4 c = ld128_stream(src + ((i + 2 * nthr) << 4));
@@ -24,8 +28,51 @@ __global__ void __launch_bounds__(1024) copy_simple_kernel(const uint8_t* __rest
         st128_stream(dst + ((i + 2 * nthr) << 4), c);
         st128_stream(dst + ((i + 3 * nthr) << 4), d);
     }
-    for (; i < nvec; i += nthr) st128_stream(dst + (i << 4), ld128_stream(src + (i << 4)));
+    for (; i < hi; i += nthr) st128_stream(dst + (i << 4), ld128_stream(src + (i << 4)));
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (tid < (nbytes & 15u)) dst[(nvec << 4) + tid] = src[(nvec << 4) + tid];
+}
+
+// Read-only pass: XOR of all whole 16-byte vectors of a buffer, folded into
+// four 32-bit words (per wavefront by lane exchange, per block through LDS,
+// then one atomic per word and block).  The HBM read-bandwidth yardstick: the
+// ring kernels read far more than they write.
+__global__ void __launch_bounds__(1024) read_xor_kernel(const uint8_t* __restrict__ src,
+                                                        uint64_t nbytes, uint32_t* out) {
+    __shared__ uint32_t part[16][4];
+    const uint64_t nvec = nbytes >> 4;
+    const uint64_t per = (nvec + gridDim.x - 1) / gridDim.x;
+    const uint64_t lo = (uint64_t)blockIdx.x * per;
+    const uint64_t hi = lo + per < nvec ? lo + per : nvec;
+    const uint64_t nthr = blockDim.x;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    uint64_t i = lo + threadIdx.x;
+    for (; i + 3 * nthr < hi; i += 4 * nthr) {
+        u32x4 a = ld128_stream(src + (i << 4));
+        u32x4 b = ld128_stream(src + ((i + nthr) << 4));
+        u32x4 c = ld128_stream(src + ((i + 2 * nthr) << 4));
+        u32x4 d = ld128_stream(src + ((i + 3 * nthr) << 4));
+        acc ^= (a ^ b) ^ (c ^ d);
+    }
+    for (; i < hi; i += nthr) acc ^= ld128_stream(src + (i << 4));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        acc.x ^= __shfl_xor(acc.x, off);
+        acc.y ^= __shfl_xor(acc.y, off);
+        acc.z ^= __shfl_xor(acc.z, off);
+        acc.w ^= __shfl_xor(acc.w, off);
+    }
+    const int wv = wave_in_block();
+    if (lane_id() == 0) {
+        part[wv][0] = acc.x; part[wv][1] = acc.y; part[wv][2] = acc.z; part[wv][3] = acc.w;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        uint32_t x = 0;
+        const int nw = (int)(blockDim.x >> 6);
+        for (int k = 0; k < nw; ++k) x ^= part[k][threadIdx.x];
+        atomicXor(out + threadIdx.x, x);
+    }
 }
 
 // ---- LL128 codec, wave64 layout: one wavefront per block -------------------

@@ -256,6 +256,26 @@ int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int 
     return launch_status();
 }
 
+int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int threads,
+                  void* stream) {
+    if (!out) return MINT_ERR_ARG;
+    if (nbytes < 16) return MINT_OK;
+    if (!src) return MINT_ERR_ARG;
+    if (!aligned16(src)) return MINT_ERR_ALIGN;
+    if (threads <= 0) threads = 512;
+    if (threads % 64 || threads > 1024) return MINT_ERR_ARG;
+    if (blocks <= 0) {
+        blocks = device_cus() * (2048 / threads);
+        if (blocks <= 0) return MINT_ERR_HIP;
+    }
+    const uint64_t need = (nbytes / 16 + (uint64_t)threads - 1) / (uint64_t)threads;
+    if ((uint64_t)blocks > need) blocks = (int)need;
+    hipLaunchKernelGGL(read_xor_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0,
+                       as_stream(stream), static_cast<const uint8_t*>(src), (uint64_t)nbytes,
+                       static_cast<uint32_t*>(out));
+    return launch_status();
+}
+
 size_t mint_ll128_packed_bytes(size_t nbytes, int layout) {
     if (layout == MINT_LAYOUT_PAIR) return (nbytes + 119) / 120 * 128;
     return (nbytes + 959) / 960 * 1024;

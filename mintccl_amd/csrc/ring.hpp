@@ -253,7 +253,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         return q;
     };
     // load_ll128 of the wave's own rows for one group: only the loads;
-    // arrange_own finishes the job where the values are needed.
+    // ll_arrange finishes the job where the values are needed.
     auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -490,9 +490,6 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const Role role = role_of(a, p, h);
     if (h == 0 && a.skip_origin) return;
 
-#ifdef MINT_RING_GENERIC_ROLE
-    ring_walk<PROTO, DT, CPI, U>(a, p, h, w, role);
-#else
     // one specialised walk per role
     const int rk = role.rank, nx = role.next;
     if (!role.recv) {
@@ -512,7 +509,6 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     } else {
         ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<false, true, false, true, false>{rk, nx});
     }
-#endif
 }
 
 }  // namespace mint

@@ -29,6 +29,20 @@ def copy128(src: torch.Tensor, dst: torch.Tensor, blocks: int = 0, threads: int 
                                                _stream(src)), "mint_copy_simple")
 
 
+def read_xor(src: torch.Tensor, out: torch.Tensor | None = None, blocks: int = 0,
+             threads: int = 0) -> torch.Tensor:
+    """XOR of all whole 16-byte vectors of ``src`` as four uint32 words (a
+    read-only pass: the HBM read-bandwidth yardstick).  ``out`` (int32[4],
+    zeroed by the caller) is XORed into; without it a fresh one is made."""
+    n = src.numel() * src.element_size()
+    if out is None:
+        out = torch.zeros(4, dtype=torch.int32, device=src.device)
+    with torch.cuda.device(src.device):
+        _lib.check(_lib.lib().mint_read_xor(src.data_ptr(), n, out.data_ptr(), blocks, threads,
+                                            _stream(src)), "mint_read_xor")
+    return out
+
+
 def Sum(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """Elementwise ``rn(a + b)``, one rounding, by the ring kernels' own adder."""
     if a.dtype not in DTYPE_CODE or a.dtype != b.dtype or a.numel() != b.numel():

@@ -43,6 +43,19 @@ def test_copy_simple(dev, n):
     assert torch.equal(dst[:n], src) and int(dst[n:].sum()) == 0
 
 
+@pytest.mark.parametrize("n", [0, 15, 16, 1000, (1 << 20) + 5, (64 << 20) + 16])
+def test_read_xor_matches_numpy(dev, n):
+    """The read-only yardstick really reads everything: its XOR of all whole
+    16-byte vectors equals numpy's."""
+    from mintccl_amd import primitive
+    g = torch.Generator().manual_seed(77 + n)
+    host = torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g)
+    got = primitive.read_xor(host.to(dev)).cpu().numpy().view(np.uint32)
+    whole = host.numpy()[: n // 16 * 16].view(np.uint32).reshape(-1, 4)
+    want = np.bitwise_xor.reduce(whole, axis=0) if len(whole) else np.zeros(4, np.uint32)
+    assert got.tolist() == want.tolist()
+
+
 @pytest.mark.parametrize("layout", [ll128.LAYOUT_PAIR, ll128.LAYOUT_WAVE64])
 @pytest.mark.parametrize("n", SIZES)
 def test_pack_unpack_match_oracle(dev, layout, n):
