@@ -167,6 +167,20 @@ int mint_elementwise_sum(const void* a, const void* b, void* out, size_t nelem, 
 size_t mint_ring_staging_bytes(const mint_ring_op* op);
 /* Blocks the launch will use; negative mint_error if the geometry is bad. */
 int mint_ring_grid_blocks(const mint_ring_op* op);
+/* The chunk schedule of one wave-channel, listed on the host by the code the
+ * kernels walk (the reference computes it inline in every kernel: sendrecv
+ * 2_sendrecv_indirect.py:61,76-77, buffered 3_sendrecv_buffer.py:32-34,46-47,
+ * reducescatter 7_reducescatter.py:23-34,43-44,75-77, allgather
+ * 6_allgather.py:42,57-59,91-102).  For wave-channel `wave` at `position`
+ * (0 = origin .. hops = sink) of `pipeline`, in the order it handles them:
+ * step[i], block[i] (block number inside the row: 960 raw bytes for LL128,
+ * 1024 for Simple), recv_offset[i] / send_offset[i] (byte offset of the
+ * block's 1 KiB message inside the staging of the rank it is received in /
+ * sent to).  Any output array may be NULL; at most max_entries are written,
+ * *n_entries is the full count.  Needs no GPU. */
+int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
+                       uint32_t max_entries, uint32_t* step, uint32_t* block,
+                       uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries);
 /* Validate and enqueue one fused launch that runs every rank's kernel. */
 int mint_ring_launch(const mint_ring_op* op, void* stream);
 

@@ -63,6 +63,7 @@ class RingOp(ctypes.Structure):
 _vp, _sz, _u64, _u32, _i = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
                             ctypes.c_uint32, ctypes.c_int)
 _ip = ctypes.POINTER(ctypes.c_int)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
 _opp = ctypes.POINTER(RingOp)
 SYMBOLS = {
     "mint_version": (_i, []),
@@ -77,6 +78,7 @@ SYMBOLS = {
     "mint_elementwise_sum": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
     "mint_ring_staging_bytes": (_sz, [_opp]),
     "mint_ring_grid_blocks": (_i, [_opp]),
+    "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
     "mint_ring_launch": (_i, [_opp, _vp]),
     "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }

@@ -205,7 +205,6 @@ __global__ void __launch_bounds__(256) torn_probe_kernel(uint8_t* staging, uint3
                                                          unsigned long long* counters) {
     const LaneMap m;
     const uint32_t wpb = blockDim.x >> 6;
-    const uint32_t pair_blocks = (pairs + wpb - 1) / wpb;
     uint32_t pb; bool producer;
     if (placement == 1) {
         // producer and consumer of a pair are consecutive blocks of the same XCD

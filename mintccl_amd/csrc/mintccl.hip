@@ -187,6 +187,36 @@ int launch_ring(const Plan& plan, int protocol, int dtype, int cache_policy, hip
     }
 }
 
+template <int U>
+int list_schedule(const RingArgs& a, uint32_t raw_per_block, int pipeline, int position, int wave,
+                  uint32_t max_entries, uint32_t* step, uint32_t* block, uint32_t* recv_offset,
+                  uint32_t* send_offset, uint32_t* n_entries) {
+    uint64_t row_bytes;
+    uint32_t nblocks, nfull;
+    row_extent(a, pipeline, raw_per_block, row_bytes, nblocks, nfull);
+    const WalkGeom geom{(uint32_t)a.waves, a.k_per_wave, a.step_blocks, a.nslots, a.slot_bytes,
+                        a.step_msg, nblocks, nfull, (uint32_t)wave};
+    const uint32_t share_recv = share_of(a, pipeline, position);
+    const uint32_t share_send = share_of(a, pipeline, position + 1);
+    const uint32_t ngroups = a.steps * (a.k_per_wave / (uint32_t)U);
+    uint32_t n = 0;
+    Group<U> q = Group<U>::first_of(geom);
+    for (uint32_t i = 0; i < ngroups; ++i, q = q.next(geom)) {
+        for (int u = 0; u < U; ++u) {
+            if (!q.valid[u]) continue;
+            if (n < max_entries) {
+                if (step) step[n] = q.step;
+                if (block) block[n] = q.g[u];
+                if (recv_offset) recv_offset[n] = q.msg_off(geom, share_recv, u);
+                if (send_offset) send_offset[n] = q.msg_off(geom, share_send, u);
+            }
+            ++n;
+        }
+    }
+    *n_entries = n;
+    return MINT_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -373,6 +403,30 @@ int mint_ring_grid_blocks(const mint_ring_op* op) {
     Plan plan;
     const int err = make_plan(op, &plan);
     return err != MINT_OK ? err : plan.blocks;
+}
+
+int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
+                       uint32_t max_entries, uint32_t* step, uint32_t* block,
+                       uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries) {
+    if (!n_entries) return MINT_ERR_ARG;
+    *n_entries = 0;
+    Plan plan;
+    const int err = make_plan(op, &plan);
+    if (err != MINT_OK) return err;
+    if (plan.empty) return MINT_OK;
+    const RingArgs& a = plan.args;
+    if (pipeline < 0 || pipeline >= a.pipes || position < 0 || position > a.hops || wave < 0 ||
+        wave >= a.waves)
+        return MINT_ERR_ARG;
+    const uint32_t raw = op->protocol == MINT_PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
+    switch (plan.unroll) {
+        case 4: return list_schedule<4>(a, raw, pipeline, position, wave, max_entries, step, block,
+                                        recv_offset, send_offset, n_entries);
+        case 2: return list_schedule<2>(a, raw, pipeline, position, wave, max_entries, step, block,
+                                        recv_offset, send_offset, n_entries);
+        default: return list_schedule<1>(a, raw, pipeline, position, wave, max_entries, step, block,
+                                         recv_offset, send_offset, n_entries);
+    }
 }
 
 int mint_ring_launch(const mint_ring_op* op, void* stream) {

@@ -143,6 +143,84 @@ __device__ __forceinline__ bool wait_count(const uint64_t* word, uint32_t epoch,
     }
 }
 
+// ---- chunk scheduler --------------------------------------------------------
+// Which blocks of its row a wave-channel moves, in which order, and where they
+// sit in a staging slot (the reference computes this inline in every kernel,
+// e.g. 7_reducescatter.py:23-34,43-44,75-77).  Host and device share this
+// code: the kernels walk it, mint_ring_schedule lists it.
+//
+// A row is cut into blocks (960 raw bytes for LL128, 1024 for Simple).  Step s
+// covers blocks [s * step_blocks, (s + 1) * step_blocks); inside a step,
+// wave-channel w of W takes blocks k * W + w, k = 0 .. K - 1, U at a time (a
+// group).  Block i of a step travels in bytes [i * 1024, (i + 1) * 1024) of
+// this (pipeline, phase)'s share of slot s mod nslots.
+struct WalkGeom {
+    uint32_t waves, k_per_wave, step_blocks, nslots, slot_bytes, step_msg;
+    uint32_t nblocks;        // blocks of this row (allreduce rows may be clipped)
+    uint32_t nfull;          // of which lie wholly inside the row
+    uint32_t w;              // this wave-channel
+};
+template <int U>
+struct Group {
+    uint32_t step, slot, k0, idx[U], g[U];
+    bool valid[U], full[U], first, last;
+    __host__ __device__ __forceinline__ void fill(const WalkGeom& s) {
+        first = k0 == 0;
+        last = k0 + (uint32_t)U >= s.k_per_wave;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            idx[u] = (k0 + (uint32_t)u) * s.waves + s.w;
+            g[u] = step * s.step_blocks + idx[u];
+            valid[u] = g[u] < s.nblocks;
+            full[u] = g[u] < s.nfull;
+        }
+    }
+    __host__ __device__ __forceinline__ static Group first_of(const WalkGeom& s) {
+        Group q;
+        q.step = 0; q.slot = 0; q.k0 = 0;
+        q.fill(s);
+        return q;
+    }
+    // The walk over (step, first block) is kept incrementally: no division.
+    __host__ __device__ __forceinline__ Group next(const WalkGeom& s) const {
+        Group q;
+        q.step = step; q.slot = slot; q.k0 = k0 + (uint32_t)U;
+        if (q.k0 >= s.k_per_wave) {
+            q.k0 = 0;
+            ++q.step;
+            q.slot = slot + 1 == s.nslots ? 0 : slot + 1;
+        }
+        q.fill(s);
+        return q;
+    }
+    // byte offset of block u of this group inside a rank's staging
+    __host__ __device__ __forceinline__ uint32_t msg_off(const WalkGeom& s, uint32_t share,
+                                                         int u) const {
+        return slot * s.slot_bytes + share * s.step_msg + idx[u] * 1024u;
+    }
+};
+// Row p of the launch: its length (allreduce splits one buffer into `world`
+// rows; the last ones may be short or empty) and its block counts.
+__host__ __device__ __forceinline__ void row_extent(const RingArgs& a, int p, uint32_t raw_per_block,
+                                                    uint64_t& row_bytes, uint32_t& nblocks,
+                                                    uint32_t& nfull) {
+    const uint64_t row_off = (uint64_t)p * a.row_stride;
+    row_bytes = a.row_bytes;
+    nblocks = a.nblocks;
+    if (a.total_bytes) {
+        const uint64_t left = a.total_bytes > row_off ? a.total_bytes - row_off : 0;
+        row_bytes = left < a.row_bytes ? left : a.row_bytes;
+        nblocks = (uint32_t)((row_bytes + raw_per_block - 1) / raw_per_block);
+    }
+    nfull = (uint32_t)(row_bytes / raw_per_block);    // these take the unguarded path
+}
+// A rank can receive twice in one pipeline of an allreduce (once while the sum
+// is built, once while it is handed round): each phase has its own share of
+// the slots and its own credit words.
+__host__ __device__ __forceinline__ uint32_t share_of(const RingArgs& a, int p, int h) {
+    return (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
+}
+
 // How staging memory is accessed.  The sector tags make any choice safe: a
 // stale or partially visible sector fails its tag test and is polled again,
 // so a wrong policy costs time (or a reported time-out), never data.
@@ -178,27 +256,15 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
     const LaneMap m;
     const uint64_t row_off = (uint64_t)p * a.row_stride;
-    // allreduce splits one buffer into `world` rows; the last ones may be short or empty
-    uint64_t row_bytes = a.row_bytes;
-    uint32_t nblocks = a.nblocks;
-    if (a.total_bytes) {
-        const uint64_t left = a.total_bytes > row_off ? a.total_bytes - row_off : 0;
-        row_bytes = left < a.row_bytes ? left : a.row_bytes;
-        const uint32_t per_block = PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple;
-        nblocks = (uint32_t)((row_bytes + per_block - 1) / per_block);
-    }
+    uint64_t row_bytes;
+    uint32_t nblocks, nfull;
+    row_extent(a, p, PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple, row_bytes, nblocks, nfull);
     const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
     uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
-    // blocks that lie wholly inside the row take the unguarded path
-    const uint32_t nfull = (uint32_t)(row_bytes / (PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple));
     const uint32_t ring_bytes = a.nslots * a.slot_bytes;
     const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
     const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);
-    // a rank can receive twice in one pipeline of an allreduce (once while
-    // the sum is built, once while it is handed round): each phase has its own
-    // share of the slots and its own credit words
-    const uint32_t share_recv = (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
-    const uint32_t share_send = (uint32_t)p * (uint32_t)a.phases + (h + 1 >= a.world && a.phases > 1 ? 1u : 0u);
+    const uint32_t share_recv = share_of(a, p, h), share_send = share_of(a, p, h + 1);
     const uint32_t own_chan = a.credit_off + (share_recv * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
     const uint32_t nxt_chan = a.credit_off + (share_send * (uint32_t)a.waves + (uint32_t)w) * kCreditStride;
     uint64_t* own_tail = reinterpret_cast<uint64_t*>(a.staging[role.rank] + own_chan);
@@ -221,37 +287,10 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
     const uint64_t t_begin = timing ? wall_clock64() : 0;
 
-    // Group = U blocks of this wave-channel inside one step.  The walk over
-    // (step, first block) is kept incrementally: no division in the loop.
-    struct Group { uint32_t step, slot, k0, idx[U], g[U]; bool valid[U], full[U], first, last; };
-    auto fill = [&](Group& q) {
-        q.first = q.k0 == 0;
-        q.last = q.k0 + (uint32_t)U >= K;
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            q.idx[u] = (q.k0 + (uint32_t)u) * W + (uint32_t)w;
-            q.g[u] = q.step * a.step_blocks + q.idx[u];
-            q.valid[u] = q.g[u] < nblocks;
-            q.full[u] = q.g[u] < nfull;
-        }
-    };
-    auto first_group = [&]() {
-        Group q;
-        q.step = 0; q.slot = 0; q.k0 = 0;
-        fill(q);
-        return q;
-    };
-    auto next_group = [&](const Group& cur) {
-        Group q;
-        q.step = cur.step; q.slot = cur.slot; q.k0 = cur.k0 + (uint32_t)U;
-        if (q.k0 >= K) {
-            q.k0 = 0;
-            ++q.step;
-            q.slot = cur.slot + 1 == a.nslots ? 0 : cur.slot + 1;
-        }
-        fill(q);
-        return q;
-    };
+    // Group = U blocks of this wave-channel inside one step
+    const WalkGeom geom{W, K, a.step_blocks, a.nslots, a.slot_bytes, a.step_msg, nblocks, nfull,
+                        (uint32_t)w};
+    using Group = mint::Group<U>;
     // load_ll128 of the wave's own rows for one group: only the loads;
     // ll_arrange finishes the job where the values are needed.
     auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
@@ -287,7 +326,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     u32x4 v[U], vnext[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
-    Group q = first_group();
+    Group q = Group::first_of(geom);
     uint32_t n = 0;
     // Loop-carried, and looked at in every iteration whether or not a credit
     // was asked for: the compiler then knows that no load into these
@@ -305,10 +344,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // the guarded body and load their own rows on the spot.
     auto run_group = [&](auto whole_tag) -> bool {
         constexpr bool WHOLE = decltype(whole_tag)::value;
-        const Group qn = next_group(q);
+        const Group qn = q.next(geom);
         const uint32_t s = q.step;
-        const uint32_t slot_off = q.slot * a.slot_bytes + share_recv * a.step_msg;
-        const uint32_t send_off = q.slot * a.slot_bytes + share_send * a.step_msg;
         const uint32_t tag = (a.epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the credit for the slot this step
         // goes into is only needed before the send, so its load is issued
@@ -332,7 +369,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 if (WHOLE || q.valid[u])
-                    r[u] = ld128<LDCP>(own, slot_off + q.idx[u] * kBlockMsg + m.lane * 16u);
+                    r[u] = ld128<LDCP>(own, q.msg_off(geom, share_recv, u) + m.lane * 16u);
         }
         if (role.load) {
             if (WHOLE) fetch_ahead(qn, vnext);
@@ -355,7 +392,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     if (!(pending & (1u << u))) continue;
-                    if (ll_poll<LDCP>(own, slot_off + q.idx[u] * kBlockMsg, tag, m, r[u]))
+                    if (ll_poll<LDCP>(own, q.msg_off(geom, share_recv, u), tag, m, r[u]))
                         pending &= ~(1u << u);
                 }
             }
@@ -398,9 +435,9 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             }
             if (role.send) {
                 if (PROTO == PROTO_LL128)
-                    ll_send<STCP>(nxt, send_off + q.idx[u] * kBlockMsg, v[u], tag, m);
+                    ll_send<STCP>(nxt, q.msg_off(geom, share_send, u), v[u], tag, m);
                 else
-                    st128<STCP>(nxt, send_off + q.idx[u] * kBlockMsg + m.lane * 16u, v[u]);
+                    st128<STCP>(nxt, q.msg_off(geom, share_send, u) + m.lane * 16u, v[u]);
             }
         }
         if (q.last) {
