@@ -36,7 +36,8 @@ extern "C" {
 typedef enum {
     MINT_OK = 0,
     MINT_ERR_ARG = -1,        /* bad argument (null, range, unknown enum) */
-    MINT_ERR_ALIGN = -2,      /* address or stride not 16-byte aligned */
+    MINT_ERR_ALIGN = -2,      /* address not 16-byte aligned (staging; buffers of the stand-alone
+                                 copy, codec and sum entry points; ring buffers need none) */
     MINT_ERR_GEOMETRY = -3,   /* slot / wave geometry does not divide */
     MINT_ERR_RESIDENCY = -4,  /* grid would not be co-resident on the device */
     MINT_ERR_HIP = -5,        /* a HIP runtime call failed */
@@ -57,15 +58,18 @@ typedef enum {
 } mint_op;
 typedef enum {
     MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
-    MINT_PLACE_LOCAL = 1    /* every hop of a channel on the same XCD */
+    MINT_PLACE_LOCAL = 1    /* every hop of a channel on the same XCD: each block takes its
+                               work from the XCD it runs on; needs a device that deals
+                               every 8 consecutive blocks to 8 different XCDs
+                               (mint_device_info reports 8, mint_xcd_map shows the order) */
 } mint_placement;
 
 /* Status block written by the ring kernel (device memory, 4 x uint64, zeroed
  * by the caller before launch).  word 0: 0 = OK, else 1 = a bounded wait ran
  * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
  * that gave up; word 2: step it waited for; word 3: abort flag polled by all
- * other waits.  Error code 2: a block did not run on XCD (block index % 8), which
- * cache_policy 2 relies on; word 2 then holds the XCD it ran on.
+ * other waits.  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
+ * then holds that number.
  * The reference has no abort path (common.py:106 is unused). */
 #define MINT_STATUS_WORDS 4
 
@@ -126,7 +130,8 @@ int mint_device_info(int* compute_units, int* xcds, int* wave_size);
 
 /* XCC_ID of the XCD each of `blocks` thread blocks of a 1-D launch lands on
  * (device uint32[blocks]); documents the block -> XCD dealing order that the
- * placement option relies on. */
+ * placement option relies on: round-robin, starting at an XCD that depends on
+ * the hardware queue behind the stream. */
 int mint_xcd_map(int blocks, void* out, void* stream);
 
 /* Simple-protocol copy, 16 bytes per lane, persistent grid.

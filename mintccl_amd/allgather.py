@@ -24,3 +24,10 @@ def allgather(buff: torch.Tensor, comm: VirtualComm | None = None) -> None:
     d = comm.make_op(_lib.OP_ALLGATHER, _lib.BYTES, row, ptrs, ptrs, ring_of(comm),
                      row_stride=row)
     comm.launch(d)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("allgather"))

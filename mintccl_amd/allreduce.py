@@ -28,3 +28,10 @@ def allreduce(buff: torch.Tensor, comm: VirtualComm | None = None) -> None:
     ptrs = {r: info["ptr"] for r, info in posted.items()}
     d = comm.make_op(_lib.OP_ALLREDUCE, dtype, count, ptrs, ptrs, ring_of(comm))
     comm.launch(d)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("allreduce"))

@@ -23,3 +23,10 @@ def broadcast(buff: torch.Tensor, root: int, comm: VirtualComm | None = None) ->
     d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, count, {root: ptrs[root]},
                      {r: p for r, p in ptrs.items() if r != root}, ring_of(comm), root=root)
     comm.launch(d)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("broadcast"))

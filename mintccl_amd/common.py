@@ -126,8 +126,23 @@ class RingTimeout(RuntimeError):
 
 
 class PlacementError(RuntimeError):
-    """cache_policy 2 was used but a block did not run on the XCD the
-    round-robin dealing predicts (status word 0 == 2)."""
+    """The local placement ran on a device that numbers its XCDs beyond 7
+    (status word 0 == 2)."""
+
+
+_XCDS: dict[int, int] = {}
+
+
+def _xcd_count(device: torch.device) -> int:
+    """XCDs the device deals thread blocks over (asked once per device)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _XCDS:
+        import ctypes
+        n = ctypes.c_int(0)
+        with torch.cuda.device(index):
+            _lib.check(_lib.lib().mint_device_info(None, ctypes.byref(n), None), "mint_device_info")
+        _XCDS[index] = n.value
+    return _XCDS[index]
 
 
 def _largest_divisor_at_most(n: int, cap: int) -> int:
@@ -179,8 +194,9 @@ class VirtualComm:
         self.slot_bytes = self.buff_size // self.nslots
         self.protocol = protocol if protocol is not None else protocol_env()
         if placement is None:
+            # the local placement deals channels to 8 XCDs: only where there are 8
             placement = placement_env() if os.getenv("MINTCCL_PLACEMENT") else (
-                _lib.PLACE_LOCAL if tuned else _lib.PLACE_SPREAD)
+                _lib.PLACE_LOCAL if tuned and _xcd_count(self.device) == 8 else _lib.PLACE_SPREAD)
         self.placement = placement
         if waves_per_rank is None:
             waves_per_rank = (max(1, num_blocks() * num_warps() // 2) if reference_geometry
@@ -356,9 +372,8 @@ class VirtualComm:
             who = st[1]
             if st[0] == 2:
                 raise PlacementError(
-                    f"block of pipeline {who >> 32}, position {(who >> 16) & 0xFFFF} ran on XCD "
-                    f"{st[2]}: thread blocks are not dealt round-robin over the XCDs here; "
-                    "use cache_policy 0")
+                    f"a block ran on XCD {st[2]}: the local placement deals work to XCDs 0..7; "
+                    "use placement spread (and cache_policy 0) on this device")
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
                 f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]}")

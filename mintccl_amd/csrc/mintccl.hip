@@ -99,8 +99,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     } else {
         a.row_bytes = op->count_bytes;
         a.row_stride = rowwise ? op->row_stride : 0;
-        if (rowwise && (op->row_stride < op->count_bytes || !aligned16(op->row_stride)))
-            return MINT_ERR_ALIGN;
+        if (rowwise && op->row_stride < op->count_bytes) return MINT_ERR_ARG;   // rows overlap
     }
     plan->empty = op->count_bytes == 0 || op->world == 1 ||
                   (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);
@@ -114,10 +113,9 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
             const bool save = allreduce ? h >= op->world - 1
                                         : sink || ((op->op == MINT_OP_BROADCAST ||
                                                     op->op == MINT_OP_ALLGATHER) && !origin);
-            if (load && (!op->input[rank] || !aligned16(op->input[rank])))
-                return op->input[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
-            if (save && (!op->output[rank] || !aligned16(op->output[rank])))
-                return op->output[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+            // caller buffers and rows may start at any byte; staging is ours
+            if (load && !op->input[rank]) return MINT_ERR_ARG;
+            if (save && !op->output[rank]) return MINT_ERR_ARG;
             if (!origin && (!op->staging[rank] || !aligned16(op->staging[rank])))
                 return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
         }
@@ -227,7 +225,7 @@ const char* mint_strerror(int err) {
     switch (err) {
         case MINT_OK: return "ok";
         case MINT_ERR_ARG: return "bad argument";
-        case MINT_ERR_ALIGN: return "address or stride not 16-byte aligned";
+        case MINT_ERR_ALIGN: return "address not 16-byte aligned";
         case MINT_ERR_GEOMETRY: return "slot / wave geometry does not divide";
         case MINT_ERR_RESIDENCY: return "grid would not be co-resident on the device";
         case MINT_ERR_HIP: return "HIP runtime call failed";

@@ -114,6 +114,15 @@ __device__ __forceinline__ u32x4 ld128_stream(const void* p) {
 __device__ __forceinline__ void st128_stream(void* p, u32x4 v) {
     __builtin_nontemporal_store(v, as_global(reinterpret_cast<u32x4*>(p)));
 }
+// The same for rows of the caller's buffers in the ring kernels, which may
+// start at any byte.
+typedef u32x4 u32x4_unaligned __attribute__((aligned(1)));
+__device__ __forceinline__ u32x4 ld128_row(const void* p) {
+    return __builtin_nontemporal_load((MINT_GLOBAL const u32x4_unaligned*)p);
+}
+__device__ __forceinline__ void st128_row(void* p, u32x4 v) {
+    __builtin_nontemporal_store(v, (MINT_GLOBAL u32x4_unaligned*)p);
+}
 __device__ __forceinline__ u32x2 ld64_stream(const void* p) {
     return __builtin_nontemporal_load(as_global(reinterpret_cast<const u32x2*>(p)));
 }

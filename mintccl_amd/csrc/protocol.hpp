@@ -26,9 +26,13 @@
 
 namespace mint {
 
-typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+// Caller rows may start at any byte: row accesses are typed with alignment 1
+// (the device runs compute queues in unaligned access mode, and the compiler
+// still emits one dwordx4 / dwordx3 / dwordx2 instruction per access).
+typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
 typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
-typedef u32x3 u32x3_a4 __attribute__((aligned(4)));
+typedef u32x3 u32x3_a1 __attribute__((aligned(1)));
+typedef u32x2 u32x2_a1 __attribute__((aligned(1)));
 
 constexpr uint32_t kLineBytes = 128, kLinePayload = 120;
 constexpr uint32_t kBlockMsg = 1024, kBlockRawLL = 960, kBlockRawSimple = 1024;
@@ -59,12 +63,12 @@ __device__ __forceinline__ u32x4 load_guarded(const uint8_t* base_, uint64_t off
     if (off >= nbytes) return v;
     uint64_t have = nbytes - off;
     if (have >= len) {
-        if (len == 16u) return *(MINT_GLOBAL const u32x4*)(base + off);
+        if (len == 16u) return *(MINT_GLOBAL const u32x4_a1*)(base + off);
         if (len == 12u) {
-            u32x3 h = *(MINT_GLOBAL const u32x3_a4*)(base + off);
+            u32x3 h = *(MINT_GLOBAL const u32x3_a1*)(base + off);
             v.x = h.x; v.y = h.y; v.z = h.z;
         } else {                                   // 8
-            u32x2 h = *(MINT_GLOBAL const u32x2*)(base + off);
+            u32x2 h = *(MINT_GLOBAL const u32x2_a1*)(base + off);
             v.x = h.x; v.y = h.y;
         }
         return v;
@@ -81,13 +85,13 @@ __device__ __forceinline__ void store_guarded(uint8_t* base_, uint64_t off, uint
     if (off >= nbytes) return;
     uint64_t have = nbytes - off;
     if (have >= len) {
-        if (len == 16u) { *(MINT_GLOBAL u32x4*)(base + off) = v; return; }
+        if (len == 16u) { *(MINT_GLOBAL u32x4_a1*)(base + off) = v; return; }
         if (len == 12u) {
             u32x3 h = {v.x, v.y, v.z};
-            *(MINT_GLOBAL u32x3_a4*)(base + off) = h;
+            *(MINT_GLOBAL u32x3_a1*)(base + off) = h;
         } else {                                   // 8
             u32x2 h = {v.x, v.y};
-            *(MINT_GLOBAL u32x2*)(base + off) = h;
+            *(MINT_GLOBAL u32x2_a1*)(base + off) = h;
         }
         return;
     }
@@ -111,7 +115,7 @@ __device__ __forceinline__ u32x4 ll_fetch_raw(const uint8_t* row, uint64_t row_b
         // 16-byte load that stays inside the block
         const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
         return __builtin_nontemporal_load(
-            (MINT_GLOBAL const u32x4_a4*)(row + base + off));
+            (MINT_GLOBAL const u32x4_a1*)(row + base + off));
     }
     return load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
 }
@@ -130,11 +134,11 @@ __device__ __forceinline__ void ll_save_raw(uint8_t* row, uint64_t row_bytes, ui
     const uint64_t base = (uint64_t)g * kBlockRawLL;
     if (full) {
         if (!m.flag_lane) {
-            st128_stream(row + base + m.raw_off, v);
+            __builtin_nontemporal_store(v, (MINT_GLOBAL u32x4_a1*)(row + base + m.raw_off));
         } else {
             u32x3 h = {v.x, v.y, v.z};
             __builtin_nontemporal_store(
-                h, (MINT_GLOBAL u32x3_a4*)(row + base + m.raw_off));
+                h, (MINT_GLOBAL u32x3_a1*)(row + base + m.raw_off));
         }
     } else {
         store_guarded(row, base + m.raw_off, m.raw_len, row_bytes, v);

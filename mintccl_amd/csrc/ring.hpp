@@ -105,7 +105,8 @@ __device__ __forceinline__ Role role_of(const RingArgs& a, int p, int h) {
 }
 
 // First wavefront that gives up records why (1 = a bounded wait ran out,
-// 2 = block not on the expected XCD) and who it was; everybody else sees word 3.
+// 2 = the local placement met an XCD number beyond 7) and who it was;
+// everybody else sees word 3.
 __device__ __forceinline__ void report_error(uint64_t* status, uint64_t code, int p, int h, int w,
                                              uint64_t detail) {
     if (lane_id() == 0) {
@@ -230,8 +231,8 @@ __host__ __device__ __forceinline__ uint32_t share_of(const RingArgs& a, int p, 
 //   2  XCD-local: stores (and credit words) carry no scope bits and stay in
 //      the L2 of the XCD; loads are agent scope, which skips the per-CU L1 and
 //      is served by that L2 while the line is still there.  Only valid with
-//      PLACE_LOCAL, where all hops of a channel share one XCD; the kernel
-//      checks that blocks really are dealt round-robin over the XCDs.
+//      PLACE_LOCAL, where all hops of a channel share one XCD (each block
+//      takes its work from the XCD it finds itself on).
 //      (Measured alternatives: nt loads behave like sc1 loads; plain and sc0
 //      loads keep hitting stale L1 lines and time out, with or without
 //      buffer_inv sc0.)
@@ -302,7 +303,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 v[u] = ll_fetch_raw(in_row, row_bytes, q.g[u], q.full[u], m);
             } else {
                 const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                v[u] = q.full[u] ? ld128_stream(in_row + off)
+                v[u] = q.full[u] ? ld128_row(in_row + off)
                                  : load_guarded(in_row, off, 16u, row_bytes);
             }
         }
@@ -319,7 +320,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             if (PROTO == PROTO_LL128)
                 v[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
             else
-                v[u] = ld128_stream(in_row + (uint64_t)g * kBlockRawSimple + m.lane * 16u);
+                v[u] = ld128_row(in_row + (uint64_t)g * kBlockRawSimple + m.lane * 16u);
         }
     };
 
@@ -429,7 +430,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     ll_save_raw(out_row, row_bytes, q.g[u], full, m, v[u]);
                 } else {
                     const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                    if (full) st128_stream(out_row + off, v[u]);
+                    if (full) st128_row(out_row + off, v[u]);
                     else store_guarded(out_row, off, 16u, row_bytes, v[u]);
                 }
             }
@@ -491,12 +492,22 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const int x = (int)blockIdx.x;
     int c, h;
     if (a.placement == PLACE_LOCAL) {
-        // blocks are dealt round-robin over the XCDs: block x runs on XCD
-        // x % 8.  Give XCD d the channels c with c % 8 == d and let the blocks
-        // it receives walk through the positions of one channel after the
-        // other, so a channel's whole ring shares one L2, is dispatched
-        // together, and every CU hosts a mix of positions.
-        const int xcd = x % kXcds, y = x / kXcds;
+        // Blocks are dealt round-robin over the XCDs, so every aligned group of
+        // 8 consecutive blocks lands on 8 different XCDs - but not always block
+        // x on XCD x % 8: which XCD block 0 goes to depends on the hardware
+        // queue the stream is mapped to (measured: 0 on a fresh process, 7 on
+        // the default stream once a second stream has been used).  So a block
+        // asks the hardware where it runs, and the group it belongs to says
+        // how far along that XCD's list of work it is: XCD d takes the
+        // channels c with c % 8 == d and its blocks walk through the
+        // positions of one channel after the other.  A channel's whole ring
+        // then shares one L2 by construction, is dispatched together, and
+        // every CU hosts a mix of positions.
+        const int xcd = xcc_id(), y = x / kXcds;
+        if (xcd >= kXcds) {
+            report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
+            return;
+        }
         h = y % npos;
         c = (y / npos) * kXcds + xcd;
     } else {
@@ -519,11 +530,6 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     int w = gw * wpb + wib;
     if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
         w = (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
-    if (CPI == 2 && xcc_id() != x % kXcds) {
-        // the XCD-local policy rests on block x running on XCD x % 8
-        report_error(a.status, 2, p, h, w, (uint64_t)xcc_id());
-        return;
-    }
     const Role role = role_of(a, p, h);
     if (h == 0 && a.skip_origin) return;
 

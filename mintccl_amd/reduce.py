@@ -26,3 +26,10 @@ def reduce(buff: torch.Tensor, root: int, comm: VirtualComm | None = None) -> No
     d = comm.make_op(_lib.OP_REDUCE, dtype, count, ptrs, {root: ptrs[root]}, ring_of(comm),
                      root=root)
     comm.launch(d)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("reduce"))

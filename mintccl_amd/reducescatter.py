@@ -28,3 +28,10 @@ def reducescatter(buff: torch.Tensor, comm: VirtualComm | None = None) -> None:
     d = comm.make_op(_lib.OP_REDUCESCATTER, dtype, row, ptrs, ptrs, ring_of(comm),
                      row_stride=row)
     comm.launch(d)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("reducescatter"))

@@ -36,3 +36,10 @@ def recv(buff: torch.Tensor, peer: int, profile: bool = True,
                                                stream), "mint_copy_simple")
     if profile:                      # 1_sendrecv_direct.py:77-79
         torch.cuda.synchronize(comm.device)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("sendrecv_direct"))

@@ -19,3 +19,10 @@ def sync(comm: VirtualComm | None = None, route: list[int] | None = None) -> Non
     s, r = st["send"], st["recv"]
     st["send"] = st["recv"] = None
     _buffered._launch(comm, s, r, route, full_size_staging=True)
+
+
+if __name__ == "__main__":      # the reference runs its self-test from here
+    import sys
+
+    from .selftest import main
+    sys.exit(main("sendrecv_indirect"))

@@ -122,8 +122,7 @@ def test_plan_geometry_without_a_gpu():
     (dict(slot_bytes=4096), _lib.ERR_GEOMETRY),        # less than one block per pipeline
     (dict(waves_per_channel_group=7), _lib.ERR_GEOMETRY),
     (dict(nslots=0), _lib.ERR_GEOMETRY),
-    (dict(row_stride=(1 << 20) + 8), _lib.ERR_ALIGN),
-    (dict(row_stride=1 << 19), _lib.ERR_ALIGN),       # rows would overlap
+    (dict(row_stride=1 << 19), _lib.ERR_ARG),         # rows would overlap
     (dict(count_bytes=(1 << 20) + 1, row_stride=1 << 21), _lib.ERR_ARG),
     (dict(slot_bytes=1 << 30, nslots=8), _lib.ERR_TOO_LARGE),
 ])
@@ -139,6 +138,10 @@ def test_plan_rejects_bad_buffers_and_rings():
     d = make_op()
     d.staging[2] += 8
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ALIGN
+    d = make_op(row_stride=(1 << 20) + 2)            # caller rows may start at any byte
+    d.input[1] += 1
+    d.output[1] += 1
+    assert L.mint_ring_grid_blocks(d) > 0
     d = make_op()
     d.ring[8] = 1                                    # ring does not close
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG

@@ -25,11 +25,28 @@ def test_device_is_mi355x_shaped(lib):
 
 
 def test_blocks_are_dealt_round_robin_over_xcds(lib, dev):
+    """What the local placement relies on: consecutive blocks go to consecutive
+    XCDs, so every aligned group of 8 covers all 8 - from whichever XCD block
+    0 lands on, which changes with the hardware queue behind the stream."""
     from mintccl_amd import primitive
     cu, xcd, wave = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     lib.mint_device_info(cu, xcd, wave)
-    m = primitive.xcd_map(64, dev).cpu().tolist()
-    assert m == [i % xcd.value for i in range(64)]
+    n = xcd.value
+
+    def check():
+        m = primitive.xcd_map(64, dev).cpu().tolist()
+        assert m == [(m[0] + i) % n for i in range(64)]
+        return m[0]
+
+    starts = {check()}
+    other = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(other):
+        src = torch.zeros(1 << 20, dtype=torch.uint8, device=dev)
+        primitive.copy128(src, torch.empty_like(src), blocks=3, threads=256)
+        starts.add(check())
+    other.synchronize()
+    starts.add(check())          # the default stream may have moved to another queue
+    assert starts <= set(range(n))
 
 
 @pytest.mark.parametrize("n", [0, 1, 16, 1000, (1 << 20) + 5, (64 << 20) + 16])

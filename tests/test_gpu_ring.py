@@ -52,13 +52,40 @@ ROW_ELEMS = [1, 8, 479, 480, 481, 4096, 100003]      # ragged, one block, many s
 @pytest.mark.parametrize("world", WORLDS)
 @pytest.mark.parametrize("n", ROW_ELEMS)
 def test_reducescatter_f16(dev, world, n):
-    if (n * 2) % 16:                 # rows of a (world, n) buffer must start 16-byte aligned
-        n = (n + 7) // 8 * 8
     host = rank_rows(world, n, "f16")
     bufs = [h.to(dev) for h in host]
     comm = make_comm(world, buff_size_=world * 8 * 8192, nslots=8, waves_per_rank=8 * world)
     run_reducescatter(comm, bufs)
     assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
+
+@pytest.mark.parametrize("proto", [0, 1])
+@pytest.mark.parametrize("shift", [1, 2, 6, 9])
+def test_buffers_and_rows_at_any_byte(dev, proto, shift):
+    """Neither the buffers nor the rows of a (world, n) tensor need any
+    alignment: buffers carved `shift` elements into an allocation, rows of an
+    odd number of elements (many full blocks and a ragged end)."""
+    from mintccl_amd.allgather import allgather
+    world, n = 4, 3 * 480 * 5 + 7
+    host = rank_rows(world, n, "f16")
+    backing = [torch.zeros(world * n + 64, dtype=torch.float16, device=dev) for _ in range(world)]
+    bufs = [b[shift: shift + world * n].view(world, n) for b in backing]
+    for b, h in zip(bufs, host):
+        b.copy_(h)
+    assert all(b.data_ptr() % 16 == (2 * shift) % 16 for b in bufs)
+    comm = make_comm(world, protocol=proto)
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+    # nothing written outside the buffers
+    for b in backing:
+        assert int(b[:shift].abs().sum()) == 0 and int(b[shift + world * n:].abs().sum()) == 0
+    for b, h in zip(bufs, host):
+        b.copy_(h)
+    comm.run(lambda r: allgather(bufs[r], comm))
+    comm.check()
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    for b in backing:
+        assert int(b[:shift].abs().sum()) == 0 and int(b[shift + world * n:].abs().sum()) == 0
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])

@@ -157,3 +157,23 @@ def test_launch_is_asynchronous_and_stream_ordered(dev):
     comm.check()
     want = host.to(dev).float().sum()
     assert torch.all(total == want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("world,count", [(8, 1 << 20), (4, (1 << 18) + 24), (2, 65536)])
+def test_reference_style_self_tests_pass(monkeypatch, capsys, world, count):
+    """MINTCCL_TEST_MODE=1 python -m mintccl_amd.<op>: every collective prints
+    `equal: True` against the same collective done with plain torch operations
+    (the reference compares with torch.distributed, 4_broadcast.py:111-126)."""
+    from mintccl_amd import selftest
+    monkeypatch.setenv("MINTCCL_TEST_MODE", "1")
+    monkeypatch.setenv("MINTCCL_TEST_COUNT", str(count))
+    monkeypatch.setenv("MINTCCL_WORLD_SIZE", str(world))
+    monkeypatch.setenv("ROOT_TEMP", str(world - 1))
+    monkeypatch.setenv("DST_TEMP", str(world - 1))
+    assert selftest.main("all") == 0
+    out = capsys.readouterr().out
+    assert "equal: False" not in out
+    # 3 point-to-point tests, broadcast and allgather and allreduce on every rank,
+    # reduce at the root, reducescatter on every rank
+    assert out.count("equal: True") == 3 + 3 * world + 1 + world
