@@ -469,3 +469,43 @@ def test_headline_reducescatter_256mib_fp16(dev):
         for k in range(1, world):
             acc = primitive.Sum(orig[(c + k) % world][c].contiguous(), acc)
         assert torch.equal(bufs[c][c].view(torch.int16), acc.view(torch.int16))
+
+
+def test_empty_buffers_are_a_no_op(dev):
+    """Zero bytes: every collective returns without launching and touches nothing."""
+    from mintccl_amd.allgather import allgather
+    from mintccl_amd.allreduce import allreduce
+    from mintccl_amd.broadcast import broadcast
+    from mintccl_amd.reduce import reduce
+    from mintccl_amd.reducescatter import reducescatter
+    world = 4
+    comm = make_comm(world)
+    rows = [torch.empty(world, 0, dtype=torch.float16, device=dev) for _ in range(world)]
+    flat = [torch.empty(0, dtype=torch.float16, device=dev) for _ in range(world)]
+    comm.run(lambda r: reducescatter(rows[r], comm))
+    comm.run(lambda r: allgather(rows[r], comm))
+    comm.run(lambda r: reduce(flat[r], 1, comm))
+    comm.run(lambda r: broadcast(flat[r], 2, comm))
+    comm.run(lambda r: allreduce(flat[r], comm))
+    comm.check()
+
+
+def test_rows_beyond_4_gib(dev):
+    """Offsets inside a row are 64-bit: a 4 GiB + 960 KiB + 40 B message through two
+    hops (rank 0 -> 1 -> 2 as a broadcast over 3 ranks) arrives bit for bit."""
+    from mintccl_amd.broadcast import broadcast
+    n = (4 << 30) + 960 * 1024 + 40
+    world = 3
+    src = torch.empty(n, dtype=torch.uint8, device=dev)
+    # a pattern that differs every 4 GiB: byte i = (i * 2654435761 >> 7) & 255 on 64-bit i
+    step = 1 << 28
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        i = torch.arange(lo, hi, dtype=torch.int64, device=dev)
+        src[lo:hi] = ((i * 2654435761) >> 7).to(torch.uint8)
+        del i
+    bufs = [src, torch.zeros(n, dtype=torch.uint8, device=dev), torch.zeros(n, dtype=torch.uint8, device=dev)]
+    comm = make_comm(world)
+    run_broadcast(comm, bufs, 0)
+    for b in bufs[1:]:
+        assert torch.equal(b, src)
