@@ -222,9 +222,11 @@ def config5(reps: int, max_log2: int) -> None:
 
 
 def allreduce_bench(reps: int) -> None:
-    """The reference's planned 8_allreduce: 8 ranks x 256 MiB fp16.  Payload
-    bytes (6N - 4) S: per chunk N own-row reads, 2N - 2 staging writes and
-    reads, N result writes."""
+    """The reference's planned 8_allreduce: 8 ranks x 256 MiB fp16, as a
+    reduce-scatter launch followed by an allgather launch (the default) and as
+    one pass round the ring.  Payload bytes (6N - 4) S for the one pass: per
+    chunk N own-row reads, 2N - 2 staging writes and reads, N result writes;
+    the same figure is used for both so that the rates compare."""
     from mintccl_amd.allreduce import allreduce
     world = 8
     for n in (33554432, 134217728):
@@ -234,12 +236,13 @@ def allreduce_bench(reps: int) -> None:
             orig.append(torch.randn(n, generator=g, device=DEV, dtype=torch.float32)
                         .to(torch.float16))
         S = n * 2
-        for name, proto in (("ll128", 0), ("simple", 1)):
+        for name, proto, fused in (("ll128", 0, False), ("ll128", 0, True), ("simple", 1, False),
+                                   ("simple", 1, True)):
             comm = comm_for(world, proto, None)
             bufs = [o.clone() for o in orig]
 
             def step():
-                comm.run(lambda r: allreduce(bufs[r], comm))
+                comm.run(lambda r: allreduce(bufs[r], comm, fused=fused))
 
             step()
             comm.check()
@@ -251,8 +254,9 @@ def allreduce_bench(reps: int) -> None:
                 ok = ok and all(torch.equal(b[c * row:(c + 1) * row].view(torch.int16),
                                             want.view(torch.int16)) for b in bufs)
             ms = time_ms(step, reps)
-            emit(config="next", op="allreduce", protocol=name, staging="tuned", world=world,
-                 bytes=S, ms=round(ms, 4), alg_gbps=round((6 * world - 4) * S / ms / 1e6, 1),
+            emit(config="next", op="allreduce", protocol=name,
+                 mode="one pass" if fused else "reducescatter + allgather", staging="tuned",
+                 world=world, bytes=S, ms=round(ms, 4), alg_gbps=round((6 * world - 4) * S / ms / 1e6, 1),
                  algbw_gbps=round(S / ms / 1e6, 1),
                  busbw_gbps=round(2 * (world - 1) / world * S / ms / 1e6, 1), ok=ok,
                  grid=comm.last_grid)

@@ -120,6 +120,13 @@ typedef struct {
                               re-polls, ticks waiting for credit, ticks
                               polling, ticks total, wavefronts, 0, 0}; a tick
                               is 10 ns.  Other builds reject non-zero. */
+    uint64_t total_bytes;  /* ALLGATHER / REDUCESCATTER: 0, or the rows are the
+                              pieces of one buffer of total_bytes bytes, cut
+                              every row_stride bytes: row p ends where the
+                              buffer ends (short or empty last rows), and
+                              count_bytes is the length of a full row.  This
+                              is how an allreduce runs as a reducescatter
+                              followed by an allgather.  Other ops: 0. */
 } mint_ring_op;
 
 int mint_version(void);

@@ -56,6 +56,7 @@ class RingOp(ctypes.Structure):
         ("status", ctypes.c_uint64),
         ("debug_skip_origin", ctypes.c_uint32), ("credit_offset", ctypes.c_uint32),
         ("debug_stats", ctypes.c_uint64),
+        ("total_bytes", ctypes.c_uint64),
     ]
 
 

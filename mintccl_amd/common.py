@@ -282,7 +282,8 @@ class VirtualComm:
     # ---- launch -------------------------------------------------------------
     def make_op(self, op: int, dtype: int, count_bytes: int, inputs: dict, outputs: dict,
                 ring: list[int], root: int = 0, row_stride: int = 0, route_len: int = 0,
-                protocol: int | None = None, skip_origin: bool = False) -> _lib.RingOp:
+                protocol: int | None = None, skip_origin: bool = False,
+                total_bytes: int = 0) -> _lib.RingOp:
         d = _lib.RingOp()
         d.op, d.dtype, d.world = op, dtype, self.world_size
         d.protocol = self.protocol if protocol is None else protocol
@@ -293,7 +294,7 @@ class VirtualComm:
             d.input[r] = inputs.get(r, NULL)
             d.output[r] = outputs.get(r, NULL)
             d.staging[r] = self.staging_ptr(r)
-        d.count_bytes, d.row_stride = count_bytes, row_stride
+        d.count_bytes, d.row_stride, d.total_bytes = count_bytes, row_stride, total_bytes
         # credit words at a fixed place, whatever slot geometry a launch uses
         d.credit_offset = self.buff_size
         pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER,

@@ -90,6 +90,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     const int dt_size = op->dtype == MINT_F32 ? 4 : (op->dtype == MINT_BYTES ? 1 : 2);
     if (op->count_bytes % dt_size) return MINT_ERR_ARG;
     if (allreduce) {
+        if (op->total_bytes) return MINT_ERR_ARG;
         // one buffer of count_bytes per rank, cut into `world` rows of whole
         // 16-byte vectors; the last rows may be short or empty
         const uint64_t per = (op->count_bytes + op->world - 1) / op->world;
@@ -100,6 +101,13 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
         a.row_bytes = op->count_bytes;
         a.row_stride = rowwise ? op->row_stride : 0;
         if (rowwise && op->row_stride < op->count_bytes) return MINT_ERR_ARG;   // rows overlap
+        if (op->total_bytes) {
+            // rows cut from one buffer: the last ones may be short or empty
+            if (!rowwise || op->total_bytes % dt_size ||
+                op->total_bytes > (uint64_t)op->world * op->row_stride)
+                return MINT_ERR_ARG;
+            a.total_bytes = op->total_bytes;
+        }
     }
     plan->empty = op->count_bytes == 0 || op->world == 1 ||
                   (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);

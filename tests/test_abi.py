@@ -123,6 +123,10 @@ def test_plan_geometry_without_a_gpu():
     (dict(waves_per_channel_group=7), _lib.ERR_GEOMETRY),
     (dict(nslots=0), _lib.ERR_GEOMETRY),
     (dict(row_stride=1 << 19), _lib.ERR_ARG),         # rows would overlap
+    (dict(total_bytes=(8 << 20) + 16), _lib.ERR_ARG), # more than world rows hold
+    (dict(total_bytes=1001), _lib.ERR_ARG),           # not whole elements
+    (dict(op=_lib.OP_REDUCE, total_bytes=4096), _lib.ERR_ARG),     # only for rows of one buffer
+    (dict(op=_lib.OP_ALLREDUCE, waves_per_channel_group=16, total_bytes=4096), _lib.ERR_ARG),
     (dict(count_bytes=(1 << 20) + 1, row_stride=1 << 21), _lib.ERR_ARG),
     (dict(slot_bytes=1 << 30, nslots=8), _lib.ERR_TOO_LARGE),
 ])

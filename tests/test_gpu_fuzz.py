@@ -64,7 +64,9 @@ def one_case(rng: random.Random, dev, case: int):
             comm.run(lambda r: broadcast(bufs[r], root, comm))
             want = ring.broadcast(raw, root)
         else:
-            comm.run(lambda r: allreduce(bufs[r].view(-1), comm))
+            fused = rng.random() < 0.5
+            what += f" fused {fused}"
+            comm.run(lambda r: allreduce(bufs[r].view(-1), comm, fused=fused))
             want = ring.allreduce(raw, dt)
     except _lib.MintError as e:
         if e.code in (_lib.ERR_GEOMETRY, _lib.ERR_RESIDENCY):

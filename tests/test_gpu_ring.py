@@ -204,44 +204,48 @@ def test_xcd_local_policy_needs_local_placement(dev):
         make_comm(8, placement=0, cache_policy=2)
 
 
-def run_allreduce(comm, bufs):
+def run_allreduce(comm, bufs, fused=False):
     from mintccl_amd.allreduce import allreduce
-    comm.run(lambda r: allreduce(bufs[r], comm))
+    comm.run(lambda r: allreduce(bufs[r], comm, fused=fused))
     comm.check()
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("world", WORLDS)
 @pytest.mark.parametrize("n", [1, 7, 8, 63, 64, 4000, 100003, (1 << 20) + 9])
-def test_allreduce_f16(dev, world, n):
-    # ragged sizes: with few elements some chunks are short or empty
+def test_allreduce_f16(dev, world, n, fused):
+    # ragged sizes: with few elements some chunks are short or empty; as one
+    # pass round the ring, and as a reduce-scatter followed by an allgather
     host = [normal(n, 3000 + r) for r in range(world)]
     bufs = [h.to(dev) for h in host]
     comm = make_comm(world)
-    run_allreduce(comm, bufs)
+    run_allreduce(comm, bufs, fused)
     want = ring.allreduce([as_bytes(h) for h in host], "f16")
     assert same(bufs, want)
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("proto,place,cp", [(0, 0, 0), (1, 0, 0), (0, 1, 2), (1, 1, 2)])
-def test_allreduce_dtypes_protocols_policies(dev, dt, proto, place, cp):
+def test_allreduce_dtypes_protocols_policies(dev, dt, proto, place, cp, fused):
     world, n = 8, 300001
     host = [normal(n, 3000 + r, TORCH_DT[dt]) for r in range(world)]
     bufs = [h.to(dev) for h in host]
     comm = make_comm(world, protocol=proto, placement=place, cache_policy=cp,
                      buff_size_=3 * 1024 * 1024, nslots=3, waves_per_rank=512)
-    run_allreduce(comm, bufs)
+    run_allreduce(comm, bufs, fused)
     assert same(bufs, ring.allreduce([as_bytes(h) for h in host], dt))
 
 
-def test_allreduce_256mib_against_device_fold(dev):
+@pytest.mark.parametrize("fused", [False, True])
+def test_allreduce_256mib_against_device_fold(dev, fused):
     from mintccl_amd import primitive
     world, n = 8, 33554432          # 64 MiB per rank
     g = torch.Generator(device=dev).manual_seed(11)
     bufs = [torch.randn(n, generator=g, device=dev, dtype=torch.float16) for _ in range(world)]
     orig = [b.clone() for b in bufs]
     comm = make_comm(world)
-    run_allreduce(comm, bufs)
+    run_allreduce(comm, bufs, fused)
     row = n // world
     for c in range(world):
         acc = orig[c][c * row:(c + 1) * row].clone()

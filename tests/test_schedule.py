@@ -108,3 +108,15 @@ def test_schedule_rejects_positions_outside_the_launch():
     for args in ((8, 0, 0), (0, 9, 0), (0, 0, 64), (-1, 0, 0)):
         assert L.mint_ring_schedule(d, *args, 0, None, None, None, None, ctypes.byref(n)) == _lib.ERR_ARG
     assert L.mint_ring_schedule(d, 0, 0, 0, 0, None, None, None, None, None) == _lib.ERR_ARG
+
+
+def test_rows_clipped_to_one_buffer():
+    """total_bytes: the rows of a reducescatter / allgather are the pieces of one
+    buffer, the last ones short or empty (how an allreduce runs as two launches)."""
+    row = 64 * 1024 + 16
+    total = 5 * row + 1000 * 2            # rows 0..4 full, row 5 has 2000 bytes, rows 6, 7 empty
+    d = make_op(count_bytes=row, row_stride=row, total_bytes=total, waves_per_channel_group=16)
+    assert _lib.lib().mint_ring_grid_blocks(d) > 0
+    for p, left in enumerate([row] * 5 + [2000, 0, 0]):
+        blocks = np.concatenate([schedule(d, p, 1, w)[1] for w in range(16)])
+        assert sorted(blocks.tolist()) == list(range(-(-left // 960)))
