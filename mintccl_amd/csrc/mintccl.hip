@@ -185,6 +185,8 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
 // The ring kernels are compiled one element type per translation unit
 // (ring_family.hip), so that the build can run them side by side.
 int launch_ring(const Plan& plan, int protocol, int dtype, int cache_policy, hipStream_t stream) {
+    // the copying collectives move bytes whatever element type the caller names
+    if (!reducing(plan.args.op)) dtype = MINT_BYTES;
     switch (dtype) {
         case MINT_F16: return launch_ring_family_f16(plan, protocol, cache_policy, stream);
         case MINT_BF16: return launch_ring_family_bf16(plan, protocol, cache_policy, stream);

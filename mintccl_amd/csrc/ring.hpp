@@ -468,8 +468,163 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         return true;
     };
 
+    // ---- whole steps, one group per step -----------------------------------
+    // s_waitcnt vmcnt retires vector-memory operations in issue order, stores
+    // included: a wait for a poll also waits for every store issued before
+    // it.  In the loop further down the stores of a step (the sends and, for
+    // the copying roles, the saves that go to HBM) are older than the next
+    // poll, so each step ends up waiting for their acknowledgement.  When a
+    // group is a whole step (k_per_wave == U, the tuned geometries) the order
+    // is turned round: the credit word and the first poll of step s + 1 are
+    // issued as soon as the tags of step s have been accepted, before step s
+    // is added, saved and sent, and the own rows of step s + 2 after that.
+    // The stores of a step are then younger than the poll the next step waits
+    // for and have a whole step to complete.  Register buffers alternate,
+    // hence two copies of the body.  Only the copying collectives run this
+    // loop (measured: sendrecv -6 %, broadcast -8 %, allgather -4 %).  A poll
+    // issued that early finds its data only if the sender is a full step
+    // ahead, which the adding collectives - every position waiting for its
+    // own rows from HBM - are not: their early polls fail and are repeated,
+    // and reducescatter lost 12 %.
+    //
+    // The compiler derives every wait from the number of memory operations
+    // issued after the one it needs and takes the smaller number where paths
+    // meet.  So nothing in the body is issued conditionally (the tail post is
+    // stored by all lanes, fetch addresses are clamped), a wave that gives up
+    // ends on the spot instead of leaving the loop, and the prologue issues
+    // exactly the queue a later step finds (stand-ins for the stores go to an
+    // unused part of this wave-channel's own credit line).
+    if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
+      if (K == (uint32_t)U && ngroups) {
+        const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
+        uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
+        if (whole_steps > a.steps) whole_steps = a.steps;
+        if (whole_steps) {
+            u32x4 rr[2][U], vv[2][U];
+            uint64_t cw[2] = {0, 0};
+            uint32_t step = 0, slot = 0;
+            auto poll_step = [&](uint32_t at_slot, u32x4 (&r)[U]) {
+                const uint32_t base = at_slot * a.slot_bytes + share_recv * a.step_msg;
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    r[u] = ld128<LDCP>(own, base + ((uint32_t)u * W + (uint32_t)w) * kBlockMsg +
+                                                m.lane * 16u);
+            };
+            auto fetch_step = [&](uint32_t of_step, u32x4 (&x)[U]) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t g = of_step * a.step_blocks + (uint32_t)u * W + (uint32_t)w;
+                    g = g < nfull ? g : nfull - 1u;      // beyond the whole blocks: any valid address
+                    x[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
+                }
+            };
+            uint64_t* const pad = own_tail + 8;
+            auto store_pad = [&]() {
+                if (STCP == CP_NONE) st64_local(pad, 0ull);
+                else st64_agent(pad, 0ull);
+            };
+            auto give_up = [&]() {
+                report_timeout(a.status, p, h, w, step);
+                __builtin_amdgcn_endpgm();
+            };
+            if (role.load) fetch_step(0, vv[0]);
+            compiler_fence();
+            if (role.send) cw[0] = ld64_agent(nxt_tail);
+            if (role.recv) poll_step(0, rr[0]);
+            compiler_fence();
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (role.save) store_pad();
+                if (role.send) store_pad();
+            }
+            if (role.recv) store_pad();
+            compiler_fence();
+            if (role.load) fetch_step(1, vv[1]);
+            auto whole_step = [&](auto phase) {
+                constexpr int B = decltype(phase)::value, B1 = B ^ 1;
+                const uint32_t next_slot = slot + 1 == a.nslots ? 0 : slot + 1;
+                const uint32_t tag = (a.epoch << 20) | (step + 1u);
+                const uint32_t need = step >= a.nslots ? step - a.nslots + 1 : 0;
+                const uint32_t recv_base = slot * a.slot_bytes + share_recv * a.step_msg;
+                const uint32_t send_base = slot * a.slot_bytes + share_send * a.step_msg;
+                if (role.recv) {
+                    uint32_t pending = 0;
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if (!wave_all(!m.flag_lane || rr[B][u].w == tag)) pending |= 1u << u;
+                    for (uint32_t spins = 0; pending; ++spins) {
+                        if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status)))
+                            give_up();
+                        __builtin_amdgcn_s_sleep(1);
+                        compiler_fence();
+                        ++n_repoll;
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            if (!(pending & (1u << u))) continue;
+                            if (ll_poll<LDCP>(own, recv_base + ((uint32_t)u * W + (uint32_t)w) * kBlockMsg,
+                                              tag, m, rr[B][u]))
+                                pending &= ~(1u << u);
+                        }
+                    }
+                }
+                ++n_groups;
+                if (role.send) {
+                    asm volatile("" : "+v"(cw[B]));
+                    if (credits_seen < need) {
+                        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(cw[B] >> 32));
+                        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)cw[B]);
+                        if (hi == a.epoch && lo >= need) credits_seen = lo;
+                        else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
+                                             a.status))
+                            give_up();
+                    }
+                }
+                // the next step's credit word and first poll go out ahead of this step's stores
+                compiler_fence();
+                if (role.send) cw[B1] = ld64_agent(nxt_tail);
+                if (role.recv) poll_step(next_slot, rr[B1]);
+                compiler_fence();
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t idx = (uint32_t)u * W + (uint32_t)w;
+                    u32x4 x = vv[B][u];
+                    if (role.load) x = ll_arrange(x, true, m);
+                    if (role.recv) {
+                        if constexpr (DT != DT_BYTES) {
+                            x = role.reduce ? ll_comp<DT>(x, rr[B][u]) : rr[B][u];
+                        } else {
+                            x = rr[B][u];
+                        }
+                    }
+                    if (role.save)
+                        ll_save_raw(out_row, row_bytes, step * a.step_blocks + idx, true, m, x);
+                    if (role.send) ll_send<STCP>(nxt, send_base + idx * kBlockMsg, x, tag, m);
+                }
+                if (role.recv) {
+                    // post_ll128 (protocol.py:183-189); every lane stores the same word
+                    if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1));
+                    else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1));
+                }
+                compiler_fence();
+                if (role.load) fetch_step(step + 2u, vv[B]);
+                slot = next_slot;
+                ++step;
+            };
+            while (step < whole_steps) {
+                whole_step(std::integral_constant<int, 0>{});
+                if (step >= whole_steps) break;
+                whole_step(std::integral_constant<int, 1>{});
+            }
+            // what is left (a ragged or partly filled last step) starts afresh
+            q.step = step; q.slot = slot; q.k0 = 0;
+            q.fill(geom);
+            n = step;
+        }
+      }
+    }
+
     // block numbers grow from group to group, so the whole groups come first
-    if (role.load && ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
+    if (role.load && n < ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
     while (n < ngroups && q.g[U - 1] < nfull)
         if (!run_group(std::true_type{})) return;
     while (n < ngroups)
