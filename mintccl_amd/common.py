@@ -130,6 +130,34 @@ class PlacementError(RuntimeError):
     (status word 0 == 2)."""
 
 
+def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
+                   max_nslots: int) -> tuple[int, int, int]:
+    """(slot_bytes, nslots, wave-channels per (pipeline, hop)) of the tuned
+    geometry for one collective: the wavefront budget spread over the
+    (pipeline, hop) groups, one 1 KiB block per wave-channel per step, whole
+    thread blocks, and a channel count the 8 XCDs divide."""
+    pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
+    real_pipes = pipes
+    if op == _lib.OP_ALLREDUCE:
+        pipes *= 2                # a slot is shared by (pipeline, phase): two phases
+    npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: world,
+            _lib.OP_ALLGATHER: world, _lib.OP_ALLREDUCE: 2 * world - 1}.get(op, world + 1)
+    receivers = max(1, min(npos - 1, world))
+    if op == _lib.OP_ALLREDUCE:
+        npos = (npos + 1) // 2    # `pipes` already counts both phases
+    # slots sized per 8 receiving ranks keep the staging of an XCD's channels
+    # (slots x receivers / 8) well inside its 4 MiB of L2
+    multi = real_pipes > 1
+    per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
+    total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
+    nslots = min(max_nslots, TUNED_NSLOTS_MULTI) if multi else max_nslots
+    slot_blocks = min(per8 * max(1, 8 // receivers), total // npos, TUNED_SLOT_BUDGET // 1024)
+    wpb = max(1, threads_per_block // 64)
+    granule = wpb * (8 // math.gcd(real_pipes, 8))
+    waves = max(granule, slot_blocks // pipes // granule * granule)
+    return pipes * waves * 1024, nslots, waves
+
+
 _XCDS: dict[int, int] = {}
 
 
@@ -302,29 +330,8 @@ class VirtualComm:
         if op == _lib.OP_ALLREDUCE:
             pipes *= 2            # a slot is shared by (pipeline, phase): two phases
         if self.auto_geometry:
-            # spread the wavefront budget over (pipeline, hop) groups; one
-            # block per wave-channel per step; whole blocks of 4 waves per XCD
-            npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: self.world_size,
-                    _lib.OP_ALLGATHER: self.world_size,
-                    _lib.OP_ALLREDUCE: 2 * self.world_size - 1}.get(op, self.world_size + 1)
-            receivers = max(1, min(npos - 1, self.world_size))
-            if op == _lib.OP_ALLREDUCE:
-                npos = (npos + 1) // 2        # `pipes` already counts both phases
-            # slots sized per 8 receiving ranks keep the staging of an XCD's
-            # channels (slots x receivers / 8) well inside its 4 MiB of L2
-            multi = pipes > 1
-            per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
-            total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
-            nslots = min(self.nslots, TUNED_NSLOTS_MULTI) if multi else self.nslots
-            slot_blocks = min(per8 * max(1, 8 // receivers), total // npos,
-                              TUNED_SLOT_BUDGET // 1024)
-            # whole thread blocks, and a channel count the 8 XCDs divide
-            real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
-            wpb = max(1, self.threads_per_block // 64)
-            granule = wpb * (8 // math.gcd(real_pipes, 8))
-            waves = max(granule, slot_blocks // pipes // granule * granule)
-            d.slot_bytes, d.nslots = pipes * waves * 1024, nslots
-            d.waves_per_channel_group = waves
+            d.slot_bytes, d.nslots, d.waves_per_channel_group = tuned_geometry(
+                op, self.world_size, route_len, self.threads_per_block, self.nslots)
         else:
             d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
             step_blocks = self.slot_bytes // 1024 // pipes

@@ -1,7 +1,7 @@
 """Host-side logic that needs no GPU: knobs and wave-count selection."""
 import pytest
 
-from mintccl_amd import common, protocol
+from mintccl_amd import _lib, common, protocol
 
 
 def test_reference_constants():
@@ -27,3 +27,36 @@ def test_env_knobs_are_read_at_call_time(monkeypatch):
                                         (512, 128, 128), (1, 5, 1)])
 def test_largest_divisor(n, cap, want):
     assert common._largest_divisor_at_most(n, cap) == want
+
+
+@pytest.mark.parametrize("world", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("op", [_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_REDUCE, _lib.OP_ALLGATHER,
+                                _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE])
+def test_tuned_geometry_is_always_launchable(op, world):
+    """Whatever the collective and the world size, the tuned geometry passes the
+    library's own plan check, deals whole channels to the 8 XCDs, fits its
+    staging budget and stays inside the wavefront budget."""
+    from tests.test_abi import make_op
+    slot, nslots, waves = common.tuned_geometry(op, world, 2, 256, common.TUNED_NSLOTS)
+    assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
+    multi = op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
+    d = make_op(op=op, world=world, slot_bytes=slot, nslots=nslots, waves_per_channel_group=waves,
+                placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2,
+                dtype=_lib.F16 if op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
+                else _lib.BYTES)
+    for i in range(9):
+        d.ring[i] = i % world if i < world else 0
+    d.ring[world] = 0
+    if op == _lib.OP_SENDRECV:
+        d.ring[0], d.ring[1] = 0, 1
+    if op == _lib.OP_ALLREDUCE:
+        d.row_stride = 0
+    blocks = _lib.lib().mint_ring_grid_blocks(d)
+    assert blocks > 0, blocks
+    assert blocks % 8 == 0
+    assert blocks * 4 <= (common.TUNED_TOTAL_WAVES_MULTI if multi else common.TUNED_TOTAL_WAVES)
+
+
+def test_headline_geometry():
+    assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
+    assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
