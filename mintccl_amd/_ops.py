@@ -23,10 +23,16 @@ def check_buffer(t: torch.Tensor, comm: VirtualComm) -> None:
 
 
 def ring_of(comm: VirtualComm) -> list[int]:
-    topo = getattr(comm, "topology", None) or uniform_topology(comm.world_size)
-    ring = find_ring(topo)
+    """The ring of the communicator's topology (searched once per topology
+    object: the search costs more than a small collective)."""
+    topo = getattr(comm, "topology", None)
+    cached = getattr(comm, "_ring_cache", None)
+    if cached is not None and cached[0] is topo:
+        return cached[1]
+    ring = find_ring(topo or uniform_topology(comm.world_size))
     if len(ring) != comm.world_size + 1:
         raise RuntimeError("topology has no ring through every rank")
+    comm._ring_cache = (topo, ring)
     return ring
 
 
