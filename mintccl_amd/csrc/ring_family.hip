@@ -32,6 +32,16 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) !=
             hipSuccess)
             return MINT_ERR_HIP;
+        // Count one wavefront per SIMD less than the query allows.  Measured:
+        // at 4 waves per block the query says 7 blocks per CU, yet from 6
+        // blocks per CU on the grid is no longer dealt out in one go and a
+        // launch takes a third longer (the query does not see the scalar
+        // registers the platform sets aside per wave for its trap handler;
+        // a build squeezed into 16 fewer registers moved the step by exactly
+        // one wave per SIMD).
+        const int waves_per_block = plan.threads / 64;
+        per_cu = (per_cu * waves_per_block - 4) / waves_per_block;
+        if (per_cu < 1) per_cu = 1;
         memo.store(per_cu, std::memory_order_relaxed);
     }
     int ncu = cus.load(std::memory_order_relaxed);

@@ -384,6 +384,26 @@ def test_residency_is_checked(dev):
     assert e.value.code == _lib.ERR_RESIDENCY
 
 
+def test_residency_limit_is_where_the_grid_stops_fitting(dev):
+    """6 blocks of 4 waves per CU are accepted, the 7th that the occupancy query
+    would allow is not: such grids were measured to run in more than one go."""
+    from mintccl_amd import _lib
+    from mintccl_amd.reducescatter import reducescatter
+    world = 8
+    bufs = [torch.zeros(world, 4096, dtype=torch.float16, device=dev) for _ in range(world)]
+    cu = torch.cuda.get_device_properties(dev).multi_processor_count
+    # blocks = 8 pipelines x 9 positions x (waves / 4): 84 waves -> 1512 blocks, 88 -> 1584
+    ok = make_comm(world, buff_size_=2 * 84 * 8 * 1024, nslots=2, waves_per_rank=84 * 8)
+    ok.run(lambda r: reducescatter(bufs[r], ok))
+    ok.check()
+    assert ok.last_grid == 1512 <= 6 * cu
+    over = make_comm(world, buff_size_=2 * 88 * 8 * 1024, nslots=2, waves_per_rank=88 * 8)
+    assert 6 * cu < 1584 <= 7 * cu
+    with pytest.raises(_lib.MintError) as e:
+        over.run(lambda r: reducescatter(bufs[r], over))
+    assert e.value.code == _lib.ERR_RESIDENCY
+
+
 def run_probe(lib, dev, pairs, iters, cp, place, per_sector):
     st = torch.zeros(pairs * (4 * 1024 + 128), dtype=torch.uint8, device=dev)
     cnt = torch.zeros(8, dtype=torch.int64, device=dev)
