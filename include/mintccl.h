@@ -132,11 +132,13 @@ typedef struct {
 int mint_version(void);
 const char* mint_strerror(int err);
 
-/* Compute units, XCDs and wavefront size of the current device. */
+/* Compute units, XCDs and wavefront size of the current device (the reference
+ * asks torch for the multiprocessor count, common.py:72; XCDs have no
+ * counterpart there). */
 int mint_device_info(int* compute_units, int* xcds, int* wave_size);
 
 /* XCC_ID of the XCD each of `blocks` thread blocks of a 1-D launch lands on
- * (device uint32[blocks]); documents the block -> XCD dealing order that the
+ * (device uint32[blocks]).  No counterpart in the reference; documents the block -> XCD dealing order that the
  * placement option relies on: round-robin, starting at an XCD that depends on
  * the hardware queue behind the stream. */
 int mint_xcd_map(int blocks, void* out, void* stream);
@@ -193,7 +195,11 @@ int mint_ring_grid_blocks(const mint_ring_op* op);
 int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
                        uint32_t max_entries, uint32_t* step, uint32_t* block,
                        uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries);
-/* Validate and enqueue one fused launch that runs every rank's kernel. */
+/* Validate and enqueue one fused launch that runs every rank's kernel: the
+ * Triton launches kernel[(NUM_BLOCKS,)](recvbuff, sendbuff, inputbuff,
+ * outputbuff, count, ...) of 2_sendrecv_indirect.py:165-166,
+ * 3_sendrecv_buffer.py:150-151, 4_broadcast.py:100-101, 5_reduce.py:120-121,
+ * 6_allgather.py:157-158 and 7_reducescatter.py:97-98, for all ranks at once. */
 int mint_ring_launch(const mint_ring_op* op, void* stream);
 
 /* Torn-line probe: `pairs` producer wavefronts each rewrite 1 KiB blocks of
