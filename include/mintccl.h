@@ -127,6 +127,12 @@ typedef struct {
                               count_bytes is the length of a full row.  This
                               is how an allreduce runs as a reducescatter
                               followed by an allgather.  Other ops: 0. */
+    uint64_t epoch_ptr;    /* 0, or the device address of a uint32 that holds
+                              the epoch: the kernel reads it there and
+                              flag_epoch is ignored.  For launches that are
+                              captured into a HIP graph and replayed: put a
+                              mint_epoch_advance on the same word in front of
+                              every launch. */
 } mint_ring_op;
 
 int mint_version(void);
@@ -201,6 +207,16 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
  * 3_sendrecv_buffer.py:150-151, 4_broadcast.py:100-101, 5_reduce.py:120-121,
  * 6_allgather.py:157-158 and 7_reducescatter.py:97-98, for all ranks at once. */
 int mint_ring_launch(const mint_ring_op* op, void* stream);
+
+/* Advances the epoch word a mint_ring_op points to with epoch_ptr (device
+ * uint32, zero before its first use): 1, 2, ..., 4095, 1, ...  Whenever the
+ * count starts over (and on first use) the kernel also zeroes
+ * staging[0, staging_bytes) - the whole staging allocation of all ranks - as
+ * the epoch contract demands.  Enqueued on `stream` like a launch; it is what
+ * makes a captured sequence of collectives replayable, because a replay then
+ * sees fresh epochs.  No counterpart in the reference (its flags restart with
+ * every launch and it clears nothing). */
+int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, void* stream);
 
 /* Torn-line probe: `pairs` producer wavefronts each rewrite 1 KiB blocks of
  * their own `iters` times; every 64-byte sector carries a tag and a payload

@@ -57,6 +57,7 @@ class RingOp(ctypes.Structure):
         ("debug_skip_origin", ctypes.c_uint32), ("credit_offset", ctypes.c_uint32),
         ("debug_stats", ctypes.c_uint64),
         ("total_bytes", ctypes.c_uint64),
+        ("epoch_ptr", ctypes.c_uint64),
     ]
 
 
@@ -81,6 +82,7 @@ SYMBOLS = {
     "mint_ring_grid_blocks": (_i, [_opp]),
     "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
     "mint_ring_launch": (_i, [_opp, _vp]),
+    "mint_epoch_advance": (_i, [_vp, _vp, _sz, _vp]),
     "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }
 

@@ -195,7 +195,8 @@ class VirtualComm:
                  buff_size_: int | None = None, nslots: int | None = None,
                  protocol: int | None = None, placement: int | None = None,
                  waves_per_rank: int | None = None, threads_per_block: int | None = None,
-                 cache_policy: int | None = None, spin_budget: int = 0) -> None:
+                 cache_policy: int | None = None, spin_budget: int = 0,
+                 device_epoch: bool | None = None) -> None:
         self.world_size = world_size if world_size is not None else world_size_env()
         if not 1 <= self.world_size <= _lib.MAX_RANKS:
             raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
@@ -251,6 +252,14 @@ class VirtualComm:
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int64, device=self.device)
         self.stats = None              # set to a zeroed int64[(hops + 1) * 8] tensor to collect wait accounting
         self.epoch = 0
+        # Launches that are captured into a HIP graph and replayed cannot carry
+        # their epoch as an argument: with device_epoch (or MINTCCL_DEVICE_EPOCH=1)
+        # it lives in device memory and every launch is preceded by a tiny
+        # kernel that advances it (and clears staging when it starts over).
+        if device_epoch is None:
+            device_epoch = bool(os.getenv("MINTCCL_DEVICE_EPOCH", ""))
+        self.epoch_word = (torch.zeros(1, dtype=torch.int32, device=self.device)
+                           if device_epoch else None)
         self._tls = threading.local()
         self._pending: dict = {}
         self._mailbox: dict = {}
@@ -361,14 +370,22 @@ class VirtualComm:
         """Enqueue on the current stream; never synchronises."""
         # sector tags hold 12 bits of epoch: when the counter wraps, staging is
         # cleared (a stream-ordered fill) so that no tag of an old launch survives
-        if self.epoch >= _lib.MAX_EPOCH:
-            self.staging.zero_()
-            self.epoch = 0
-        self.epoch += 1
-        d.flag_epoch = self.epoch
+        if self.epoch_word is None:
+            if self.epoch >= _lib.MAX_EPOCH:
+                self.staging.zero_()
+                self.epoch = 0
+            self.epoch += 1
+            d.flag_epoch = self.epoch
+        else:
+            d.flag_epoch, d.epoch_ptr = 0, self.epoch_word.data_ptr()
         self.last_grid = self._lib.mint_ring_grid_blocks(d)
         with torch.cuda.device(self.device):
             stream = torch.cuda.current_stream().cuda_stream
+            if self.epoch_word is not None:
+                _lib.check(self._lib.mint_epoch_advance(
+                    self.epoch_word.data_ptr(), self.staging.data_ptr(),
+                    self.staging.numel() * self.staging.element_size(), stream),
+                    "mint_epoch_advance")
             _lib.check(self._lib.mint_ring_launch(d, stream), "mint_ring_launch")
 
     def check(self) -> None:

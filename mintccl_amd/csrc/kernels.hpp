@@ -33,6 +33,26 @@ __global__ void __launch_bounds__(1024) copy_simple_kernel(const uint8_t* __rest
     if (tid < (nbytes & 15u)) dst[(nvec << 4) + tid] = src[(nvec << 4) + tid];
 }
 
+// Advances a launch epoch kept in device memory: 1, 2, ..., max_epoch, 1, ...
+// and clears the staging memory whenever it starts over, so that no sector
+// tag of an earlier launch with the same number survives.  One block: the
+// clearing happens once in max_epoch launches.
+__global__ void __launch_bounds__(1024) epoch_advance_kernel(uint32_t* epoch_word, uint8_t* staging,
+                                                             uint64_t staging_bytes,
+                                                             uint32_t max_epoch) {
+    const uint32_t cur = *epoch_word;
+    __syncthreads();
+    uint32_t next = cur + 1u;
+    if (cur == 0u || cur >= max_epoch) {      // first use, or the tags are about to repeat
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        for (uint64_t i = threadIdx.x; i < (staging_bytes >> 4); i += blockDim.x)
+            *reinterpret_cast<u32x4*>(staging + (i << 4)) = zero;
+        next = 1u;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) *epoch_word = next;
+}
+
 // Read-only pass: XOR of all whole 16-byte vectors of a buffer, folded into
 // four 32-bit words (per wavefront by lane exchange, per block through LDS,
 // then one atomic per word and block).  The HBM read-bandwidth yardstick: the

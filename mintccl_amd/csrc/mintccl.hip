@@ -37,7 +37,12 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     // XCD-local staging only makes sense when every hop of a channel shares an XCD
     if (op->cache_policy == 2 && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
     if (op->placement != MINT_PLACE_SPREAD && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
-    if (op->flag_epoch == 0 || op->flag_epoch > kMaxEpoch || !op->status) return MINT_ERR_ARG;
+    if (!op->status) return MINT_ERR_ARG;
+    if (op->epoch_ptr) {
+        if (op->epoch_ptr % 4) return MINT_ERR_ALIGN;        // the epoch lives in device memory
+    } else if (op->flag_epoch == 0 || op->flag_epoch > kMaxEpoch) {
+        return MINT_ERR_ARG;
+    }
     if (op->threads_per_block == 0 || op->threads_per_block % 64 || op->threads_per_block > 512)
         return MINT_ERR_ARG;
     if (op->nslots == 0 || op->slot_bytes == 0) return MINT_ERR_GEOMETRY;
@@ -159,6 +164,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
         a.credit_off = op->credit_offset;
     }
     a.epoch = op->flag_epoch;
+    a.epoch_word = reinterpret_cast<const uint32_t*>(op->epoch_ptr);
     a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
     a.status = reinterpret_cast<uint64_t*>(op->status);
     a.skip_origin = op->debug_skip_origin;
@@ -443,6 +449,15 @@ int mint_ring_launch(const mint_ring_op* op, void* stream) {
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
     return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, as_stream(stream));
+}
+
+int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, void* stream) {
+    if (!epoch_word || (reinterpret_cast<uint64_t>(epoch_word) & 3u)) return MINT_ERR_ARG;
+    if (staging_bytes && (!staging || !aligned16(staging) || staging_bytes % 16)) return MINT_ERR_ALIGN;
+    hipLaunchKernelGGL(epoch_advance_kernel, dim3(1), dim3(1024), 0, as_stream(stream),
+                       static_cast<uint32_t*>(epoch_word), static_cast<uint8_t*>(staging),
+                       (uint64_t)staging_bytes, kMaxEpoch);
+    return launch_status();
 }
 
 int mint_torn_line_probe(void* staging, size_t staging_bytes, int pairs, int iters,

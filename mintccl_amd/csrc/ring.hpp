@@ -68,6 +68,7 @@ struct RingArgs {
     uint32_t k_per_wave;                  // step_blocks / waves
     uint32_t credit_off;                  // offset of the credit words in staging
     uint32_t epoch, spin_budget;
+    const uint32_t* epoch_word;           // optional: take the epoch from device memory instead
     uint64_t* status;
     uint32_t skip_origin;
     uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
@@ -273,7 +274,13 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + nxt_chan);
     uint64_t* nxt_head = nxt_tail + 16;
 
-    const uint64_t flag_hi = (uint64_t)a.epoch << 32;      // credit / head words
+    // The epoch normally is a launch argument; a caller that replays captured
+    // launches keeps it in device memory and advances it between launches.
+    const uint32_t epoch =
+        a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
+                           as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                     : a.epoch;
+    const uint64_t flag_hi = (uint64_t)epoch << 32;        // credit / head words
     const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
     const uint32_t groups_per_step = K / U;
     const uint32_t ngroups = a.steps * groups_per_step;
@@ -347,7 +354,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         constexpr bool WHOLE = decltype(whole_tag)::value;
         const Group qn = q.next(geom);
         const uint32_t s = q.step;
-        const uint32_t tag = (a.epoch << 20) | (s + 1u);
+        const uint32_t tag = (epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the credit for the slot this step
         // goes into is only needed before the send, so its load is issued
         // here, ahead of the polls, and looked at after them.
@@ -356,7 +363,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         if (ask_credit) credit_word = ld64_agent(nxt_tail);
         if (q.first && PROTO == PROTO_SIMPLE && role.recv) {
             const uint64_t t0 = timing ? wall_clock64() : 0;
-            if (!wait_count(own_head, a.epoch, s + 1, head_seen, a.spin_budget, a.status)) {
+            if (!wait_count(own_head, epoch, s + 1, head_seen, a.spin_budget, a.status)) {
                 report_timeout(a.status, p, h, w, s);
                 return false;
             }
@@ -404,9 +411,9 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             const uint64_t t0 = timing ? wall_clock64() : 0;
             const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(credit_word >> 32));
             const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)credit_word);
-            if (hi == a.epoch && lo >= need) {
+            if (hi == epoch && lo >= need) {
                 credits_seen = lo;
-            } else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
+            } else if (!wait_count(nxt_tail, epoch, need, credits_seen, a.spin_budget,
                                    a.status)) {
                 report_timeout(a.status, p, h, w, s);
                 return false;
@@ -543,7 +550,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             auto whole_step = [&](auto phase) {
                 constexpr int B = decltype(phase)::value, B1 = B ^ 1;
                 const uint32_t next_slot = slot + 1 == a.nslots ? 0 : slot + 1;
-                const uint32_t tag = (a.epoch << 20) | (step + 1u);
+                const uint32_t tag = (epoch << 20) | (step + 1u);
                 const uint32_t need = step >= a.nslots ? step - a.nslots + 1 : 0;
                 const uint32_t recv_base = slot * a.slot_bytes + share_recv * a.step_msg;
                 const uint32_t send_base = slot * a.slot_bytes + share_send * a.step_msg;
@@ -573,8 +580,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     if (credits_seen < need) {
                         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(cw[B] >> 32));
                         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)cw[B]);
-                        if (hi == a.epoch && lo >= need) credits_seen = lo;
-                        else if (!wait_count(nxt_tail, a.epoch, need, credits_seen, a.spin_budget,
+                        if (hi == epoch && lo >= need) credits_seen = lo;
+                        else if (!wait_count(nxt_tail, epoch, need, credits_seen, a.spin_budget,
                                              a.status))
                             give_up();
                     }

@@ -117,6 +117,7 @@ def test_plan_geometry_without_a_gpu():
     (dict(debug_stats=0x1000), _lib.ERR_ARG),            # this build collects no wait accounting
     (dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, waves_per_channel_group=16),
      _lib.ERR_GEOMETRY),                                 # 4 channels cannot be dealt to 8 XCDs
+    (dict(flag_epoch=0, epoch_ptr=0x50000002), _lib.ERR_ALIGN),   # epoch word in device memory
     (dict(threads_per_block=100), _lib.ERR_ARG),
     (dict(slot_bytes=(512 << 10) + 512), _lib.ERR_GEOMETRY),
     (dict(slot_bytes=4096), _lib.ERR_GEOMETRY),        # less than one block per pipeline
@@ -142,6 +143,7 @@ def test_plan_rejects_bad_buffers_and_rings():
     d = make_op()
     d.staging[2] += 8
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ALIGN
+    assert L.mint_ring_grid_blocks(make_op(flag_epoch=0, epoch_ptr=0x50000000)) > 0
     d = make_op(row_stride=(1 << 20) + 2)            # caller rows may start at any byte
     d.input[1] += 1
     d.output[1] += 1

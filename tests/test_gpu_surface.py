@@ -5,7 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from tests.helpers import as_bytes, normal, uniform
+from oracle import ring
+from tests.helpers import as_bytes, normal, rank_rows, uniform
 
 pytestmark = pytest.mark.gpu
 
@@ -177,3 +178,74 @@ def test_reference_style_self_tests_pass(monkeypatch, capsys, world, count):
     # 3 point-to-point tests, broadcast and allgather and allreduce on every rank,
     # reduce at the root, reducescatter on every rank
     assert out.count("equal: True") == 3 + 3 * world + 1 + world
+
+
+@pytest.mark.gpu
+def test_device_epoch_wraps_and_clears(dev):
+    """With the epoch in device memory every launch advances it; when it starts
+    over the staging is cleared, so results stay right across the wrap."""
+    from mintccl_amd.reducescatter import reducescatter
+    world, n = 4, 3000
+    comm = make_comm(world, device_epoch=True)
+    host = rank_rows(world, n, "f16")
+    want = ring.reducescatter([as_bytes(h) for h in host], "f16")
+    bufs = [h.to(dev) for h in host]
+    seen = []
+    for i in range(6):
+        if i == 2:
+            comm.epoch_word.fill_(4094)          # two launches before the count starts over
+        for b, h in zip(bufs, host):
+            b.copy_(h)
+        comm.run(lambda r: reducescatter(bufs[r], comm))
+        comm.check()
+        seen.append(int(comm.epoch_word.item()))
+        assert all(np.array_equal(as_bytes(b), w) for b, w in zip(bufs, want)), i
+    assert seen == [1, 2, 4095, 1, 2, 3]
+
+
+@pytest.mark.gpu
+def test_captured_collectives_replay(dev):
+    """A captured sequence of collectives (epoch in device memory) is replayed
+    several times, with eager work and fresh inputs in between; every replay
+    must equal the eager result."""
+    from mintccl_amd.allgather import allgather
+    from mintccl_amd.allreduce import allreduce
+    from mintccl_amd.broadcast import broadcast
+    world, n = 8, 4096 + 24
+    comm = make_comm(world, device_epoch=True)
+    eager = make_comm(world)
+    ins = [torch.zeros(world, n, dtype=torch.float16, device=dev) for _ in range(world)]
+    a = [torch.zeros_like(x) for x in ins]
+    b = [torch.zeros(world * n, dtype=torch.float16, device=dev) for _ in range(world)]
+    c = [torch.zeros(n, dtype=torch.float16, device=dev) for _ in range(world)]
+
+    def sequence(cm, a, b, c):
+        for r in range(world):
+            a[r].copy_(ins[r]); b[r].copy_(ins[r].view(-1)); c[r].copy_(ins[r][r])
+        cm.run(lambda r: allgather(a[r], cm))
+        cm.run(lambda r: allreduce(b[r], cm))
+        cm.run(lambda r: broadcast(c[r], 3, cm))
+
+    def fill(seed):
+        for r, h in enumerate(rank_rows(world, n, "f16", seed0=seed)):
+            ins[r].copy_(h.to(dev))
+
+    fill(100)
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        sequence(comm, a, b, c)                   # warm up outside the capture
+    side.synchronize()
+    comm.check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sequence(comm, a, b, c)
+    ea, eb, ec = [torch.zeros_like(x) for x in a], [torch.zeros_like(x) for x in b], [torch.zeros_like(x) for x in c]
+    for replay in range(5):
+        fill(200 + 10 * replay)
+        sequence(eager, ea, eb, ec)
+        eager.check()
+        graph.replay()
+        torch.cuda.synchronize()
+        comm.check()
+        for r in range(world):
+            assert torch.equal(a[r], ea[r]) and torch.equal(b[r], eb[r]) and torch.equal(c[r], ec[r]), replay
