@@ -10,7 +10,8 @@
  *  - plain C types only; device addresses are void* / uint64_t, 0 = absent;
  *  - every function returns 0 on success or a negative mint_error; none throws;
  *  - all work is enqueued on the hipStream_t passed as void* (NULL = the
- *    default stream); no call synchronises with the host;
+ *    default stream); no call synchronises with the host, with one exception:
+ *    mint_device_info asked for the XCD count (see there);
  *  - the caller owns every buffer and keeps it alive until the stream drains;
  *  - the library keeps no per-call state: calls on different streams are
  *    independent as long as their buffers are.
@@ -41,7 +42,8 @@ typedef enum {
     MINT_ERR_GEOMETRY = -3,   /* slot / wave geometry does not divide */
     MINT_ERR_RESIDENCY = -4,  /* grid would not be co-resident on the device */
     MINT_ERR_HIP = -5,        /* a HIP runtime call failed */
-    MINT_ERR_TOO_LARGE = -6   /* a row does not fit a 32-bit offset window */
+    MINT_ERR_TOO_LARGE = -6,  /* a row does not fit a 32-bit offset window */
+    MINT_ERR_STAGING = -7     /* staging_bytes is smaller than mint_ring_staging_bytes() */
 } mint_error;
 
 typedef enum { MINT_LAYOUT_PAIR = 0, MINT_LAYOUT_WAVE64 = 1 } mint_layout;
@@ -63,6 +65,19 @@ typedef enum {
                                every 8 consecutive blocks to 8 different XCDs
                                (mint_device_info reports 8, mint_xcd_map shows the order) */
 } mint_placement;
+
+typedef enum {
+    MINT_FETCH_INLINE = 0,  /* every wave-channel loads its own rows itself, one
+                               group ahead, into registers */
+    MINT_FETCH_LDS = 1      /* reducing ops on LL128: one more wavefront per thread
+                               block streams the own rows of the block's
+                               wave-channels from HBM into LDS several groups
+                               ahead and the wave-channels read them there, so
+                               that a poll of staging never queues behind an HBM
+                               fetch (vector-memory loads of one wavefront
+                               return in issue order).  Ignored by the ops and
+                               the protocol that have no such kernel. */
+} mint_row_fetch;
 
 /* Status block written by the ring kernel (device memory, 4 x uint64, zeroed
  * by the caller before launch).  word 0: 0 = OK, else 1 = a bounded wait ran
@@ -89,6 +104,11 @@ typedef struct {
     uint64_t input[MINT_MAX_RANKS];   /* per rank; 0 = absent */
     uint64_t output[MINT_MAX_RANKS];  /* per rank; 0 = absent */
     uint64_t staging[MINT_MAX_RANKS]; /* per rank, mint_ring_staging_bytes() each */
+    uint64_t staging_bytes; /* bytes the caller allocated behind every staging[r];
+                              a launch whose slots and credit words would not
+                              fit is refused with MINT_ERR_STAGING (the credit
+                              words sit behind the slots, outside a buffer
+                              that only holds nslots * slot_bytes) */
     uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE: bytes of the
                               buffer; ALLGATHER/REDUCESCATTER: bytes of one row */
     uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER: bytes between rows */
@@ -107,19 +127,13 @@ typedef struct {
                               memory was last zeroed */
     uint32_t spin_budget;  /* polls before a wait gives up; 0 = default */
     uint64_t status;       /* device address of MINT_STATUS_WORDS uint64 */
-    uint32_t debug_skip_origin; /* testing: origin hop sends nothing */
+    int32_t row_fetch;     /* mint_row_fetch: who reads the ranks' own rows */
     uint32_t credit_offset; /* byte offset of the credit words inside each rank's
                                staging; 0 = right after the slots.  A caller
                                that changes slot geometry between launches on
                                the same staging keeps this fixed (beyond its
                                largest nslots * slot_bytes, multiple of 256) so
                                that credit words and payload never share bytes */
-    uint64_t debug_stats;  /* 0.  A library built with -DMINT_RING_STATS takes
-                              the device address of (hops + 1) x 8 zeroed
-                              uint64 and fills, per position, {groups,
-                              re-polls, ticks waiting for credit, ticks
-                              polling, ticks total, wavefronts, 0, 0}; a tick
-                              is 10 ns.  Other builds reject non-zero. */
     uint64_t total_bytes;  /* ALLGATHER / REDUCESCATTER: 0, or the rows are the
                               pieces of one buffer of total_bytes bytes, cut
                               every row_stride bytes: row p ends where the
@@ -140,7 +154,11 @@ const char* mint_strerror(int err);
 
 /* Compute units, XCDs and wavefront size of the current device (the reference
  * asks torch for the multiprocessor count, common.py:72; XCDs have no
- * counterpart there). */
+ * counterpart there).  Any pointer may be NULL.  Asking for `xcds` is the one
+ * call of this library that allocates and synchronises: it runs a 64-block
+ * probe on the default stream and waits for it - a set-up call, not one for a
+ * serving loop or a stream under capture (mint_xcd_map is the asynchronous
+ * form). */
 int mint_device_info(int* compute_units, int* xcds, int* wave_size);
 
 /* XCC_ID of the XCD each of `blocks` thread blocks of a 1-D launch lands on
@@ -207,6 +225,20 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
  * 3_sendrecv_buffer.py:150-151, 4_broadcast.py:100-101, 5_reduce.py:120-121,
  * 6_allgather.py:157-158 and 7_reducescatter.py:97-98, for all ranks at once. */
 int mint_ring_launch(const mint_ring_op* op, void* stream);
+
+/* Test hooks, kept out of the descriptor.  skip_origin != 0: the origin hop of
+ * every pipeline sends nothing, so every other wait runs out (exercises the
+ * bounded waits and the status block).  stats: 0, or - in a library built
+ * with -DMINT_RING_STATS only, others refuse it - the device address of
+ * (hops + 1) x 8 zeroed uint64 that receive, per position, {groups, re-polls,
+ * ticks waiting for credit, ticks polling, ticks total, wavefronts, 0, 0}; a
+ * tick is 10 ns.  No counterpart in the reference. */
+typedef struct {
+    uint32_t skip_origin;
+    uint32_t reserved0;
+    uint64_t stats;
+} mint_ring_debug;
+int mint_ring_launch_debug(const mint_ring_op* op, const mint_ring_debug* dbg, void* stream);
 
 /* Advances the epoch word a mint_ring_op points to with epoch_ptr (device
  * uint32, zero before its first use): 1, 2, ..., 4095, 1, ...  Whenever the

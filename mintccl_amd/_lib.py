@@ -22,12 +22,14 @@ MAX_RANKS = 8
 STATUS_WORDS = 4
 MAX_EPOCH = 4095          # sector tags carry a 12-bit launch epoch
 
-OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE = 0, -1, -2, -3, -4, -5, -6
+(OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE,
+ ERR_STAGING) = 0, -1, -2, -3, -4, -5, -6, -7
 LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
 F16, BF16, F32, BYTES = 0, 1, 2, 3
 PROTO_LL128, PROTO_SIMPLE = 0, 1
 OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER, OP_ALLREDUCE = range(6)
 PLACE_SPREAD, PLACE_LOCAL = 0, 1
+FETCH_INLINE, FETCH_LDS = 0, 1
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -47,6 +49,7 @@ class RingOp(ctypes.Structure):
         ("input", ctypes.c_uint64 * MAX_RANKS),
         ("output", ctypes.c_uint64 * MAX_RANKS),
         ("staging", ctypes.c_uint64 * MAX_RANKS),
+        ("staging_bytes", ctypes.c_uint64),
         ("count_bytes", ctypes.c_uint64), ("row_stride", ctypes.c_uint64),
         ("slot_bytes", ctypes.c_uint32), ("nslots", ctypes.c_uint32),
         ("waves_per_channel_group", ctypes.c_uint32),
@@ -54,11 +57,16 @@ class RingOp(ctypes.Structure):
         ("placement", ctypes.c_int32), ("cache_policy", ctypes.c_int32),
         ("flag_epoch", ctypes.c_uint32), ("spin_budget", ctypes.c_uint32),
         ("status", ctypes.c_uint64),
-        ("debug_skip_origin", ctypes.c_uint32), ("credit_offset", ctypes.c_uint32),
-        ("debug_stats", ctypes.c_uint64),
+        ("row_fetch", ctypes.c_int32), ("credit_offset", ctypes.c_uint32),
         ("total_bytes", ctypes.c_uint64),
         ("epoch_ptr", ctypes.c_uint64),
     ]
+
+
+class RingDebug(ctypes.Structure):
+    """``mint_ring_debug``: the test hooks of ``mint_ring_launch_debug``."""
+    _fields_ = [("skip_origin", ctypes.c_uint32), ("reserved0", ctypes.c_uint32),
+                ("stats", ctypes.c_uint64)]
 
 
 # name -> (restype, argtypes); every symbol include/mintccl.h declares
@@ -67,6 +75,7 @@ _vp, _sz, _u64, _u32, _i = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint64,
 _ip = ctypes.POINTER(ctypes.c_int)
 _u32p = ctypes.POINTER(ctypes.c_uint32)
 _opp = ctypes.POINTER(RingOp)
+_dbgp = ctypes.POINTER(RingDebug)
 SYMBOLS = {
     "mint_version": (_i, []),
     "mint_strerror": (ctypes.c_char_p, [_i]),
@@ -82,6 +91,7 @@ SYMBOLS = {
     "mint_ring_grid_blocks": (_i, [_opp]),
     "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
     "mint_ring_launch": (_i, [_opp, _vp]),
+    "mint_ring_launch_debug": (_i, [_opp, _dbgp, _vp]),
     "mint_epoch_advance": (_i, [_vp, _vp, _sz, _vp]),
     "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }

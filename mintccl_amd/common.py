@@ -252,6 +252,7 @@ class VirtualComm:
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int64, device=self.device)
         self.stats = None              # set to a zeroed int64[(hops + 1) * 8] tensor to collect wait accounting
         self.epoch = 0
+        self._last_protocol = None
         # Launches that are captured into a HIP graph and replayed cannot carry
         # their epoch as an argument: with device_epoch (or MINTCCL_DEVICE_EPOCH=1)
         # it lives in device memory and every launch is preceded by a tiny
@@ -331,6 +332,7 @@ class VirtualComm:
             d.input[r] = inputs.get(r, NULL)
             d.output[r] = outputs.get(r, NULL)
             d.staging[r] = self.staging_ptr(r)
+        d.staging_bytes = self.rank_stride
         d.count_bytes, d.row_stride, d.total_bytes = count_bytes, row_stride, total_bytes
         # credit words at a fixed place, whatever slot geometry a launch uses
         d.credit_offset = self.buff_size
@@ -362,12 +364,25 @@ class VirtualComm:
                 d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
-        d.debug_skip_origin = int(skip_origin)
-        d.debug_stats = self.stats.data_ptr() if self.stats is not None else NULL
+        # test hooks travel beside the descriptor (mint_ring_launch_debug)
+        d.debug = None
+        if skip_origin or self.stats is not None:
+            d.debug = _lib.RingDebug(int(skip_origin), 0,
+                                     self.stats.data_ptr() if self.stats is not None else NULL)
         return d
 
     def launch(self, d: _lib.RingOp) -> None:
         """Enqueue on the current stream; never synchronises."""
+        # The Simple protocol writes raw payload where LL128 keeps its sector
+        # tags: payload left behind by a Simple launch could pass for the tags
+        # of a later LL128 launch, so the slots are cleared (a stream-ordered
+        # fill) when an LL128 launch follows a Simple one on this staging.
+        own_staging = d.staging[0] == self.staging_ptr(0)
+        if own_staging:
+            if d.protocol == _lib.PROTO_LL128 and self._last_protocol == _lib.PROTO_SIMPLE:
+                self.staging.zero_()
+                self.epoch = 0
+            self._last_protocol = d.protocol
         # sector tags hold 12 bits of epoch: when the counter wraps, staging is
         # cleared (a stream-ordered fill) so that no tag of an old launch survives
         if self.epoch_word is None:
@@ -386,7 +401,11 @@ class VirtualComm:
                     self.epoch_word.data_ptr(), self.staging.data_ptr(),
                     self.staging.numel() * self.staging.element_size(), stream),
                     "mint_epoch_advance")
-            _lib.check(self._lib.mint_ring_launch(d, stream), "mint_ring_launch")
+            if getattr(d, "debug", None) is not None:
+                _lib.check(self._lib.mint_ring_launch_debug(d, d.debug, stream),
+                           "mint_ring_launch_debug")
+            else:
+                _lib.check(self._lib.mint_ring_launch(d, stream), "mint_ring_launch")
 
     def check(self) -> None:
         """Synchronise and raise ``RingTimeout`` if a wait gave up."""

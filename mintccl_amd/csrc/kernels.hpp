@@ -53,6 +53,17 @@ __global__ void __launch_bounds__(1024) epoch_advance_kernel(uint32_t* epoch_wor
     if (threadIdx.x == 0) *epoch_word = next;
 }
 
+// Clears [p, p + nbytes), whole 16-byte vectors, with a grid-stride fill.  It
+// stands where a memset on the stream would: a fill kernel can be captured
+// into a HIP graph and replayed, a memset node cannot be relied on there.
+__global__ void __launch_bounds__(256) zero_kernel(uint8_t* p, uint64_t nbytes) {
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const uint64_t nvec = nbytes >> 4;
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += nthr)
+        *reinterpret_cast<u32x4*>(p + (i << 4)) = zero;
+}
+
 // Read-only pass: XOR of all whole 16-byte vectors of a buffer, folded into
 // four 32-bit words (per wavefront by lane exchange, per block through LDS,
 // then one atomic per word and block).  The HBM read-bandwidth yardstick: the

@@ -25,8 +25,11 @@ bool reducing(int op) {
     return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE;
 }
 
-// Everything the launch derives from the descriptor.
-int make_plan(const mint_ring_op* op, Plan* plan) {
+// Everything the launch derives from the descriptor.  `for_launch`: also
+// check what only matters once the kernels run (the size of the staging the
+// caller allocated); the host-side queries do without.
+int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
+              const mint_ring_debug* dbg = nullptr) {
     if (!op || !plan) return MINT_ERR_ARG;
     if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLREDUCE) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
@@ -37,6 +40,7 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     // XCD-local staging only makes sense when every hop of a channel shares an XCD
     if (op->cache_policy == 2 && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
     if (op->placement != MINT_PLACE_SPREAD && op->placement != MINT_PLACE_LOCAL) return MINT_ERR_ARG;
+    if (op->row_fetch != MINT_FETCH_INLINE && op->row_fetch != MINT_FETCH_LDS) return MINT_ERR_ARG;
     if (!op->status) return MINT_ERR_ARG;
     if (op->epoch_ptr) {
         if (op->epoch_ptr % 4) return MINT_ERR_ALIGN;        // the epoch lives in device memory
@@ -167,11 +171,11 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     a.epoch_word = reinterpret_cast<const uint32_t*>(op->epoch_ptr);
     a.spin_budget = op->spin_budget ? op->spin_budget : kDefaultSpinBudget;
     a.status = reinterpret_cast<uint64_t*>(op->status);
-    a.skip_origin = op->debug_skip_origin;
+    a.skip_origin = dbg ? dbg->skip_origin : 0u;
 #ifdef MINT_RING_STATS
-    a.stats = reinterpret_cast<uint64_t*>(op->debug_stats);
+    a.stats = dbg ? reinterpret_cast<uint64_t*>(dbg->stats) : nullptr;
 #else
-    if (op->debug_stats) return MINT_ERR_ARG;   // this build does not collect wait accounting
+    if (dbg && dbg->stats) return MINT_ERR_ARG;   // this build does not collect wait accounting
     a.stats = nullptr;
 #endif
     a.placement = op->placement;
@@ -185,6 +189,13 @@ int make_plan(const mint_ring_op* op, Plan* plan) {
     if (op->placement == MINT_PLACE_LOCAL && (a.pipes * a.blocks_per_group) % kXcds)
         return MINT_ERR_GEOMETRY;
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
+    plan->staging_need = (size_t)a.credit_off +
+                         (size_t)a.pipes * (size_t)a.phases * (size_t)a.waves * kCreditStride;
+    // The credit words lie behind the slots: a buffer that only holds the
+    // slots (the reference's recvbuff is BUFF_SIZE bytes, 7_reducescatter.py:93)
+    // would be written out of bounds.
+    if (for_launch && !plan->empty && op->staging_bytes < plan->staging_need)
+        return MINT_ERR_STAGING;
     return MINT_OK;
 }
 
@@ -246,6 +257,7 @@ const char* mint_strerror(int err) {
         case MINT_ERR_RESIDENCY: return "grid would not be co-resident on the device";
         case MINT_ERR_HIP: return "HIP runtime call failed";
         case MINT_ERR_TOO_LARGE: return "size does not fit the kernel's 32-bit counters";
+        case MINT_ERR_STAGING: return "staging_bytes is smaller than mint_ring_staging_bytes()";
         default: return "unknown error";
     }
 }
@@ -406,11 +418,14 @@ int mint_elementwise_sum(const void* a, const void* b, void* out, size_t nelem, 
 }
 
 size_t mint_ring_staging_bytes(const mint_ring_op* op) {
+    if (!op) return 0;
+    // asked before the staging exists: absent addresses do not matter here
+    mint_ring_op d = *op;
+    for (int r = 0; r < MINT_MAX_RANKS; ++r)
+        if (!d.staging[r]) d.staging[r] = 16;
     Plan plan;
-    if (make_plan(op, &plan) != MINT_OK) return 0;
-    return (size_t)plan.args.credit_off +
-           (size_t)plan.args.pipes * (size_t)plan.args.phases * (size_t)plan.args.waves *
-               kCreditStride;
+    if (make_plan(&d, &plan) != MINT_OK) return 0;
+    return plan.staging_need;
 }
 
 int mint_ring_grid_blocks(const mint_ring_op* op) {
@@ -444,8 +459,12 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
 }
 
 int mint_ring_launch(const mint_ring_op* op, void* stream) {
+    return mint_ring_launch_debug(op, nullptr, stream);
+}
+
+int mint_ring_launch_debug(const mint_ring_op* op, const mint_ring_debug* dbg, void* stream) {
     Plan plan;
-    const int err = make_plan(op, &plan);
+    const int err = make_plan(op, &plan, true, dbg);
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
     return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, as_stream(stream));

@@ -13,6 +13,7 @@ namespace mint {
 struct Plan {
     RingArgs args;
     int blocks, threads, unroll;
+    size_t staging_need;      // bytes of staging per rank: slots + credit words
     bool empty;
 };
 

@@ -62,6 +62,7 @@ def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None,
         comm._indirect_staging = hops
         for k in range(comm.world_size):
             d.staging[k] = hops.data_ptr() + k * per_rank
+        d.staging_bytes = per_rank
         d.credit_offset = 0                      # right after this staging's own slots
     comm.launch(d)
 

@@ -35,7 +35,7 @@ def test_version_and_strerror():
     L = _lib.lib()
     assert L.mint_version() >= 100
     assert L.mint_strerror(0) == b"ok"
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         assert L.mint_strerror(code) not in (b"ok", b"unknown error")
     assert L.mint_strerror(-99) == b"unknown error"
 
@@ -55,6 +55,22 @@ def test_descriptor_layout_matches_the_header(tmp_path):
     assert out[0] == ctypes.sizeof(_lib.RingOp)
     for f, off in zip(fields, out[1:]):
         assert getattr(_lib.RingOp, f).offset == off, f
+
+
+def test_debug_struct_layout_matches_the_header(tmp_path):
+    src = tmp_path / "layout.c"
+    fields = [f for f, _ in _lib.RingDebug._fields_]
+    lines = ["#include <stdio.h>", "#include <stddef.h>", f'#include "{HEADER}"',
+             "int main(void){", '  printf("%zu\\n", sizeof(mint_ring_debug));']
+    lines += [f'  printf("%zu\\n", offsetof(mint_ring_debug, {f}));' for f in fields]
+    lines += ["  return 0;", "}"]
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c11", "-o", str(exe), str(src)])
+    out = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert out[0] == ctypes.sizeof(_lib.RingDebug)
+    for f, off in zip(fields, out[1:]):
+        assert getattr(_lib.RingDebug, f).offset == off, f
 
 
 def test_packed_bytes():
@@ -114,7 +130,7 @@ def test_plan_geometry_without_a_gpu():
     (dict(cache_policy=2, placement=0), _lib.ERR_ARG),   # XCD-local staging needs the local placement
     (dict(credit_offset=4096), _lib.ERR_GEOMETRY),       # inside the slots
     (dict(credit_offset=(4 << 20) + 100), _lib.ERR_GEOMETRY),
-    (dict(debug_stats=0x1000), _lib.ERR_ARG),            # this build collects no wait accounting
+    (dict(row_fetch=2), _lib.ERR_ARG),
     (dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, waves_per_channel_group=16),
      _lib.ERR_GEOMETRY),                                 # 4 channels cannot be dealt to 8 XCDs
     (dict(flag_epoch=0, epoch_ptr=0x50000002), _lib.ERR_ALIGN),   # epoch word in device memory
@@ -154,6 +170,24 @@ def test_plan_rejects_bad_buffers_and_rings():
     d = make_op()
     d.ring[3] = 2                                    # rank 2 twice
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+
+
+def test_launch_refuses_undersized_staging_before_touching_the_gpu():
+    # The credit words lie behind the slots: a caller that allocates only
+    # nslots * slot_bytes (the reference's recvbuff, 7_reducescatter.py:93)
+    # is turned away instead of being written out of bounds.  The check comes
+    # before any HIP call, so it runs without a GPU.
+    L = _lib.lib()
+    d = make_op()
+    need = L.mint_ring_staging_bytes(d)
+    assert need == (4 << 20) + 8 * 16 * 256
+    for have in (0, 4 << 20, need - 1):
+        d.staging_bytes = have
+        assert L.mint_ring_launch(d, None) == _lib.ERR_STAGING
+    # a library built without wait accounting refuses a stats address
+    d.staging_bytes = need
+    dbg = _lib.RingDebug(0, 0, 0x1000)
+    assert L.mint_ring_launch_debug(d, dbg, None) == _lib.ERR_ARG
 
 
 def test_missing_library_fails_loudly(tmp_path):

@@ -238,7 +238,7 @@ def test_allreduce_dtypes_protocols_policies(dev, dt, proto, place, cp, fused):
 
 
 @pytest.mark.parametrize("fused", [False, True])
-def test_allreduce_256mib_against_device_fold(dev, fused):
+def test_allreduce_64mib_against_device_fold(dev, fused):
     from mintccl_amd import primitive
     world, n = 8, 33554432          # 64 MiB per rank
     g = torch.Generator(device=dev).manual_seed(11)
@@ -351,6 +351,38 @@ def test_payload_that_looks_like_credit_words_is_harmless(dev):
         rs = [h.to(dev) for h in host]
         run_reducescatter(comm, rs)
         assert same(rs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
+
+def test_simple_payload_that_looks_like_ll128_tags_is_harmless(dev):
+    # The Simple protocol writes raw payload into the bytes where LL128 keeps
+    # its sector tags.  A Simple broadcast whose every 32-bit word is the tag
+    # the next LL128 launch expects in step 0 must not make that launch accept
+    # stale slots: with the origin withheld, every position still has to run
+    # out of patience in step 0 (staging is cleared when LL128 follows Simple).
+    from mintccl_amd import _lib
+    from mintccl_amd.common import RingTimeout
+    world, n32 = 4, 1 << 18
+    comm = make_comm(world, spin_budget=2000)
+    ring4 = [0, 1, 2, 3, 0]
+    bufs = [torch.zeros(n32, dtype=torch.int32, device=dev) for _ in range(world)]
+    # the LL128 launch below is the first after the clearing: epoch 1, step 0
+    forged = (1 << 20) | 1
+    bufs[0].fill_(forged)
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n32 * 4, {0: ptrs[0]},
+                     {r: ptrs[r] for r in range(1, world)}, ring4, root=0,
+                     protocol=_lib.PROTO_SIMPLE)
+    comm.launch(d)
+    comm.check()
+    for b in bufs:
+        assert torch.all(b == forged)
+    d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n32 * 4, {0: ptrs[0]},
+                     {r: ptrs[r] for r in range(1, world)}, ring4, root=0,
+                     protocol=_lib.PROTO_LL128, skip_origin=True)
+    comm.launch(d)
+    assert comm.epoch == 1
+    with pytest.raises(RingTimeout, match="step 0"):
+        comm.check()
 
 
 def test_a_lost_producer_times_out_instead_of_hanging(dev):
