@@ -42,7 +42,9 @@ typedef enum {
     MINT_ERR_GEOMETRY = -3,   /* slot / wave geometry does not divide */
     MINT_ERR_RESIDENCY = -4,  /* grid would not be co-resident on the device */
     MINT_ERR_HIP = -5,        /* a HIP runtime call failed */
-    MINT_ERR_TOO_LARGE = -6,  /* a row does not fit a 32-bit offset window */
+    MINT_ERR_TOO_LARGE = -6,  /* a row does not fit a 32-bit offset window; or, for
+                                 mint_ring_launch_static, the geometry does not fit
+                                 the library's static scratch array */
     MINT_ERR_STAGING = -7     /* staging_bytes is smaller than mint_ring_staging_bytes() */
 } mint_error;
 
@@ -239,6 +241,34 @@ typedef struct {
     uint64_t stats;
 } mint_ring_debug;
 int mint_ring_launch_debug(const mint_ring_op* op, const mint_ring_debug* dbg, void* stream);
+
+/* mint_ring_launch for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference (whose host functions allocate their
+ * staging with torch on every call, e.g. 7_reducescatter.py:93).
+ * The descriptor is the one of mint_ring_launch, except that staging[],
+ * staging_bytes, credit_offset, flag_epoch and epoch_ptr are ignored: slots,
+ * credit words and the launch epoch live in a static device array inside the
+ * library, MINT_STATIC_SCRATCH_BYTES on every GPU the library runs on, held
+ * until the process ends.  The caller still passes input[], output[] and
+ * status.  Every rank gets MINT_STATIC_RANK_BYTES of it: a geometry with
+ * nslots * slot_bytes > MINT_STATIC_SLOT_BYTES or with more than
+ * MINT_STATIC_CHANNELS wave-channels per rank (pipelines x phases x
+ * waves_per_channel_group) is refused with MINT_ERR_TOO_LARGE.
+ * The call enqueues, on `stream`, a kernel that advances the epoch kept in the
+ * array (and clears the array when the 12-bit count starts over), a clearing
+ * kernel when an LL128 launch follows a Simple one, and the ring launch; it
+ * calls no hipMalloc / hipFree and no allocating library routine.  All calls
+ * on a GPU share that GPU's array: two calls that overlap in time on one GPU
+ * (different streams, or threads) race - keep them on one stream.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress) with
+ * that device current. */
+#define MINT_STATIC_SCRATCH_BYTES (16u << 20)
+#define MINT_STATIC_HEADER_BYTES 4096u
+#define MINT_STATIC_RANK_BYTES ((MINT_STATIC_SCRATCH_BYTES - MINT_STATIC_HEADER_BYTES) / MINT_MAX_RANKS)
+#define MINT_STATIC_CHANNELS 1024u
+#define MINT_STATIC_SLOT_BYTES (MINT_STATIC_RANK_BYTES - MINT_STATIC_CHANNELS * 256u)
+int mint_ring_launch_static(const mint_ring_op* op, void* stream);
 
 /* Advances the epoch word a mint_ring_op points to with epoch_ptr (device
  * uint32, zero before its first use): 1, 2, ..., 4095, 1, ...  Whenever the

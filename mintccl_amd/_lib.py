@@ -92,6 +92,7 @@ SYMBOLS = {
     "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
     "mint_ring_launch": (_i, [_opp, _vp]),
     "mint_ring_launch_debug": (_i, [_opp, _dbgp, _vp]),
+    "mint_ring_launch_static": (_i, [_opp, _vp]),
     "mint_epoch_advance": (_i, [_vp, _vp, _sz, _vp]),
     "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }

@@ -10,6 +10,15 @@
 
 using namespace mint;
 
+// Staging for mint_ring_launch_static: slots, credit words and the launch epoch
+// of all ranks, in device memory that exists from the moment the library is
+// loaded.  Every GPU the library runs on holds its own copy at its own
+// address.  In host code the name `scratch` only identifies the symbol; the
+// device address comes from hipGetSymbolAddress, once per device.
+//   [0, 4096)                              header: word 0 = launch epoch
+//   4096 + r * MINT_STATIC_RANK_BYTES      rank r: [slots ... | credit words (last 256 KiB)]
+static __device__ __align__(256) unsigned char scratch[MINT_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 constexpr int kVersion = 100;   // 0.1.0
@@ -210,6 +219,41 @@ int launch_ring(const Plan& plan, int protocol, int dtype, int cache_policy, hip
         case MINT_F32: return launch_ring_family_f32(plan, protocol, cache_policy, stream);
         default: return launch_ring_family_bytes(plan, protocol, cache_policy, stream);
     }
+}
+
+// ---- the launch that allocates nothing ---------------------------------------
+constexpr int kMaxDevices = 64;
+constexpr size_t kStaticHeader = MINT_STATIC_HEADER_BYTES;
+constexpr size_t kStaticRank = MINT_STATIC_RANK_BYTES;
+constexpr size_t kStaticSlots = MINT_STATIC_SLOT_BYTES;
+static_assert(kStaticRank % 256 == 0 && kStaticSlots % 256 == 0, "credit words are 256-byte lines");
+static_assert(kStaticHeader + MINT_MAX_RANKS * kStaticRank <= MINT_STATIC_SCRATCH_BYTES, "layout");
+
+struct StaticScratch {
+    std::atomic<unsigned char*> ptr{nullptr};   // device address of `scratch` on this device
+    std::atomic<int> last_protocol{-1};         // protocol of the previous launch on it
+};
+StaticScratch g_static[kMaxDevices];
+
+// Device address of this device's copy of `scratch` (looked up on the first
+// call with that device current).
+int static_scratch(int* dev_out, unsigned char** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MINT_ERR_HIP;
+    if (dev < 0 || dev >= kMaxDevices) return MINT_ERR_ARG;
+    unsigned char* p = g_static[dev].ptr.load(std::memory_order_acquire);
+    if (!p) {
+        void* q = nullptr;
+        if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) {
+            (void)hipGetLastError();
+            return MINT_ERR_HIP;
+        }
+        p = static_cast<unsigned char*>(q);
+        g_static[dev].ptr.store(p, std::memory_order_release);
+    }
+    *dev_out = dev;
+    *out = p;
+    return MINT_OK;
 }
 
 template <int U>
@@ -468,6 +512,51 @@ int mint_ring_launch_debug(const mint_ring_op* op, const mint_ring_debug* dbg, v
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
     return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, as_stream(stream));
+}
+
+int mint_ring_launch_static(const mint_ring_op* op, void* stream) {
+    if (!op) return MINT_ERR_ARG;
+    // size limits first: they need no device
+    if ((uint64_t)op->nslots * op->slot_bytes > kStaticSlots) return MINT_ERR_TOO_LARGE;
+    mint_ring_op d = *op;
+    d.credit_offset = (uint32_t)kStaticSlots;
+    d.staging_bytes = kStaticRank;
+    d.flag_epoch = 0;
+    d.epoch_ptr = 16;                 // stand-in until the address is known: any aligned non-zero value
+    for (int r = 0; r < MINT_MAX_RANKS; ++r) d.staging[r] = 16;
+    Plan plan;
+    int err = make_plan(&d, &plan, true);
+    if (err == MINT_ERR_STAGING) return MINT_ERR_TOO_LARGE;    // more credit words than the array holds
+    if (err != MINT_OK) return err;
+    if (plan.empty) return MINT_OK;
+
+    int dev = 0;
+    unsigned char* base = nullptr;     // device address; never the array's name
+    err = static_scratch(&dev, &base);
+    if (err != MINT_OK) return err;
+    for (int r = 0; r < MINT_MAX_RANKS; ++r)
+        plan.args.staging[r] = reinterpret_cast<uint64_t>(base + kStaticHeader + r * kStaticRank);
+    uint32_t* epoch_word = reinterpret_cast<uint32_t*>(base);
+    plan.args.epoch_word = epoch_word;
+
+    // The array keeps what the last call left in it.  The epoch in its first
+    // word makes old sector tags and credit words meaningless to this launch;
+    // the kernel that advances it clears the array on first use and whenever
+    // the 12-bit count starts over.  Raw payload of a Simple launch could pass
+    // for LL128 tags, so the slots are cleared between the two (a fill
+    // kernel, which a caller may capture, not a memset).
+    hipStream_t s = as_stream(stream);
+    const int before = g_static[dev].last_protocol.exchange(op->protocol, std::memory_order_acq_rel);
+    if (op->protocol == MINT_PROTO_LL128 && before == MINT_PROTO_SIMPLE) {
+        hipLaunchKernelGGL(zero_kernel, dim3(256), dim3(256), 0, s, base + kStaticHeader,
+                           (uint64_t)(MINT_STATIC_SCRATCH_BYTES - kStaticHeader));
+        if ((err = launch_status()) != MINT_OK) return err;
+    }
+    hipLaunchKernelGGL(epoch_advance_kernel, dim3(1), dim3(1024), 0, s, epoch_word,
+                       base + kStaticHeader, (uint64_t)(MINT_STATIC_SCRATCH_BYTES - kStaticHeader),
+                       kMaxEpoch);
+    if ((err = launch_status()) != MINT_OK) return err;
+    return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, s);
 }
 
 int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, void* stream) {
