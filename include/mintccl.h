@@ -183,6 +183,21 @@ int mint_copy_simple(const void* src, void* dst, size_t nbytes, int blocks, int 
 int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int threads,
                   void* stream);
 
+/* The memory traffic of the ring kernels' inner loop without the ring: `waves`
+ * wavefronts each run `iters` steps of, as `what` selects (bits),
+ *   1  a 16-byte-per-lane streaming load of the wave's own 960-byte block from
+ *      `rows` (block i * waves + w in step i: needs waves * iters * 960 bytes),
+ *   2  a 16-byte-per-lane agent-scope load of 1 KiB from one of the wave's two
+ *      private slots in `staging` (needs waves * 2048 bytes, 16-byte aligned),
+ *   4  a 16-byte-per-lane store of the f16 sum of the two into the other slot,
+ * with no flags and nobody waiting for anybody.  The launch takes what the
+ * device needs for that mix of accesses however well a ring schedules them:
+ * the yardstick beside mint_copy_simple and mint_read_xor.  `sink` (device
+ * uint32, may hold anything) is only written when no store is selected.  No
+ * counterpart in the reference. */
+int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
+                  int waves, int iters, int what, void* sink, void* stream);
+
 /* Standalone LL128 codec (load_ll128 + send_ll128 / recv_ll128 + save_ll128,
  * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride:
  * MINT_LAYOUT_PAIR is the reference's wire format (120 payload bytes, then the

@@ -83,6 +83,7 @@ SYMBOLS = {
     "mint_xcd_map": (_i, [_i, _vp, _vp]),
     "mint_copy_simple": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "mint_read_xor": (_i, [_vp, _sz, _vp, _i, _i, _vp]),
+    "mint_step_mix": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _vp, _vp]),
     "mint_ll128_packed_bytes": (_sz, [_sz, _i]),
     "mint_ll128_pack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp]),
     "mint_ll128_unpack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp, _vp]),

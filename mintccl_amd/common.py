@@ -63,6 +63,11 @@ def placement_env() -> int:
         os.getenv("MINTCCL_PLACEMENT", "spread").lower()]
 
 
+def row_fetch_env() -> int:
+    return {"inline": _lib.FETCH_INLINE, "lds": _lib.FETCH_LDS}[
+        os.getenv("MINTCCL_ROW_FETCH", "inline").lower()]
+
+
 def test_mode() -> bool:        # common.py:113 (any non-empty string enables it)
     return bool(os.getenv("MINTCCL_TEST_MODE", ""))
 
@@ -131,7 +136,7 @@ class PlacementError(RuntimeError):
 
 
 def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
-                   max_nslots: int) -> tuple[int, int, int]:
+                   max_nslots: int, fetcher_waves: bool = False) -> tuple[int, int, int]:
     """(slot_bytes, nslots, wave-channels per (pipeline, hop)) of the tuned
     geometry for one collective: the wavefront budget spread over the
     (pipeline, hop) groups, one 1 KiB block per wave-channel per step, whole
@@ -150,9 +155,13 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
     multi = real_pipes > 1
     per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
     total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
+    wpb = max(1, threads_per_block // 64)
+    if fetcher_waves:
+        # every thread block carries one more wavefront (it streams own rows
+        # into LDS) and a CU takes whole blocks: 24 wavefronts per CU, 256 CUs
+        total = (24 // (wpb + 1)) * 256 * wpb
     nslots = min(max_nslots, TUNED_NSLOTS_MULTI) if multi else max_nslots
     slot_blocks = min(per8 * max(1, 8 // receivers), total // npos, TUNED_SLOT_BUDGET // 1024)
-    wpb = max(1, threads_per_block // 64)
     granule = wpb * (8 // math.gcd(real_pipes, 8))
     waves = max(granule, slot_blocks // pipes // granule * granule)
     return pipes * waves * 1024, nslots, waves
@@ -196,7 +205,7 @@ class VirtualComm:
                  protocol: int | None = None, placement: int | None = None,
                  waves_per_rank: int | None = None, threads_per_block: int | None = None,
                  cache_policy: int | None = None, spin_budget: int = 0,
-                 device_epoch: bool | None = None) -> None:
+                 device_epoch: bool | None = None, row_fetch: int | None = None) -> None:
         self.world_size = world_size if world_size is not None else world_size_env()
         if not 1 <= self.world_size <= _lib.MAX_RANKS:
             raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
@@ -240,6 +249,7 @@ class VirtualComm:
         if self.cache_policy == 2 and self.placement != _lib.PLACE_LOCAL:
             raise ValueError("the XCD-local cache policy needs the local placement")
         self.spin_budget = spin_budget
+        self.row_fetch = row_fetch if row_fetch is not None else row_fetch_env()
         self._lib = _lib.lib()          # fails loudly if the extension is missing
         # slots + credit words (never more than slot_bytes / 4), zeroed: flag 0
         # and credit 0 mean "nothing yet" (2_sendrecv_indirect.py:59-60).
@@ -341,8 +351,11 @@ class VirtualComm:
         if op == _lib.OP_ALLREDUCE:
             pipes *= 2            # a slot is shared by (pipeline, phase): two phases
         if self.auto_geometry:
+            lds = (self.row_fetch == _lib.FETCH_LDS and d.protocol == _lib.PROTO_LL128
+                   and op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
+                   and self.threads_per_block // 64 in (4, 7))
             d.slot_bytes, d.nslots, d.waves_per_channel_group = tuned_geometry(
-                op, self.world_size, route_len, self.threads_per_block, self.nslots)
+                op, self.world_size, route_len, self.threads_per_block, self.nslots, lds)
         else:
             d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
             step_blocks = self.slot_bytes // 1024 // pipes
@@ -353,6 +366,7 @@ class VirtualComm:
                 step_blocks, max(1, self.waves_per_rank // pipes))
         d.threads_per_block = self.threads_per_block
         d.placement, d.cache_policy = self.placement, self.cache_policy
+        d.row_fetch = self.row_fetch
         if self.placement == _lib.PLACE_LOCAL:
             # whole channels are dealt to the 8 XCDs; when the channel count
             # does not divide, this launch runs spread with agent-scope staging

@@ -106,6 +106,37 @@ __global__ void __launch_bounds__(1024) read_xor_kernel(const uint8_t* __restric
     }
 }
 
+// ---- the memory traffic of a ring step, without the ring ---------------------
+// Every wavefront runs `iters` steps; in a step it loads its own 960-byte block
+// from `rows` the way the ring kernels do (streaming, flag lanes 4 bytes early),
+// loads 1 KiB from one of its two private slots in `staging` with the loads
+// the polls use, adds, and stores 1 KiB into the other slot - whichever of the
+// three `what` selects.  Nobody waits for anybody: the launch takes what the
+// device needs for that mix of accesses, the yardstick the ring kernels are
+// measured against.
+template <int WHAT>
+__global__ void __launch_bounds__(256) step_mix_kernel(const uint8_t* __restrict__ rows,
+                                                       uint8_t* staging, uint32_t staging_bytes,
+                                                       uint32_t waves, uint32_t iters,
+                                                       uint32_t* sink) {
+    const LaneMap m;
+    const uint32_t wave = blockIdx.x * (blockDim.x >> 6) + (uint32_t)wave_in_block();
+    if (wave >= waves) return;
+    const Window win(staging, staging_bytes);
+    const uint32_t slot0 = wave * 2u * kBlockMsg;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (uint32_t i = 0; i < iters; ++i) {
+        u32x4 own = {0u, 0u, 0u, 0u}, got = {0u, 0u, 0u, 0u};
+        if (WHAT & 2) got = ld128<CP_SC1>(win, slot0 + (i & 1u) * kBlockMsg + m.lane * 16u);
+        if (WHAT & 1) own = ll_fetch_raw(rows, 0, i * waves + wave, true, m);
+        const u32x4 x = add_rn<DT_F16>(own, got);
+        if (WHAT & 4) st128<CP_NONE>(win, slot0 + ((i + 1u) & 1u) * kBlockMsg + m.lane * 16u, x);
+        else acc ^= x;
+    }
+    if (!(WHAT & 4) && acc.x == 0x9E3779B9u && acc.y == 0x85EBCA6Bu && acc.z == 0xC2B2AE35u)
+        sink[0] = acc.w;     // keeps the loads alive; practically never taken
+}
+
 // ---- LL128 codec, wave64 layout: one wavefront per block -------------------
 __global__ void __launch_bounds__(256) pack_wave64_kernel(const uint8_t* __restrict__ raw,
                                                           uint8_t* __restrict__ msg,

@@ -25,6 +25,7 @@ constexpr int kVersion = 100;   // 0.1.0
 constexpr uint32_t kDefaultSpinBudget = 4000000u;
 constexpr uint32_t kMaxEpoch = 4095u;          // 12 bits of every sector tag
 constexpr uint32_t kMaxSteps = (1u << 20) - 1; // 20 bits of every sector tag
+constexpr uint32_t kFetchDepth = 4;            // own rows through LDS: groups of LDS per wave-channel
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
@@ -191,7 +192,15 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
 
     const int waves_per_block = (int)op->threads_per_block / 64;
     plan->threads = (int)op->threads_per_block;
-    if (a.waves < waves_per_block) plan->threads = a.waves * 64;
+    // Own rows through LDS: LL128 reductions, thread blocks of 4 or 7
+    // wave-channels (plus the fetcher), one or two blocks per wave-channel and
+    // step.  Everything else runs the walk that fetches its rows itself.
+    a.k_per_wave = a.step_blocks / (uint32_t)a.waves;
+    plan->lds = op->row_fetch == MINT_FETCH_LDS && op->protocol == MINT_PROTO_LL128 &&
+                reducing(op->op) && (waves_per_block == 4 || waves_per_block == 7) &&
+                a.k_per_wave % 4 != 0;
+    a.fetch_depth = plan->lds ? kFetchDepth : 0u;
+    if (!plan->lds && a.waves < waves_per_block) plan->threads = a.waves * 64;
     a.blocks_per_group = (a.waves * 64 + plan->threads - 1) / plan->threads;
     plan->blocks = a.pipes * (a.hops + 1) * a.blocks_per_group;
     // the XCD-local mapping deals whole channels to XCDs
@@ -373,6 +382,34 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
     hipLaunchKernelGGL(read_xor_kernel, dim3((unsigned)blocks), dim3((unsigned)threads), 0,
                        as_stream(stream), static_cast<const uint8_t*>(src), (uint64_t)nbytes,
                        static_cast<uint32_t*>(out));
+    return launch_status();
+}
+
+int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
+                  int waves, int iters, int what, void* sink, void* stream) {
+    if (waves <= 0 || iters <= 0 || what < 1 || what > 7) return MINT_ERR_ARG;
+    if ((what & 1) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
+        return MINT_ERR_ARG;
+    if ((size_t)waves * (size_t)iters >= (1ull << 32)) return MINT_ERR_TOO_LARGE;
+    if ((what & 6) && (!staging || staging_bytes < (size_t)waves * 2u * kBlockMsg)) return MINT_ERR_ARG;
+    if ((what & 6) && staging_bytes >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
+    if ((what & 6) && !aligned16(staging)) return MINT_ERR_ALIGN;
+    if (!(what & 4) && !sink) return MINT_ERR_ARG;
+    void (*kernel)(const uint8_t*, uint8_t*, uint32_t, uint32_t, uint32_t, uint32_t*) = nullptr;
+    switch (what) {
+        case 1: kernel = step_mix_kernel<1>; break;
+        case 2: kernel = step_mix_kernel<2>; break;
+        case 3: kernel = step_mix_kernel<3>; break;
+        case 4: kernel = step_mix_kernel<4>; break;
+        case 5: kernel = step_mix_kernel<5>; break;
+        case 6: kernel = step_mix_kernel<6>; break;
+        default: kernel = step_mix_kernel<7>; break;
+    }
+    const unsigned blocks = ((unsigned)waves + 3u) / 4u;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint8_t*>(rows), static_cast<uint8_t*>(staging),
+                       (uint32_t)staging_bytes, (uint32_t)waves, (uint32_t)iters,
+                       static_cast<uint32_t*>(sink));
     return launch_status();
 }
 

@@ -72,6 +72,7 @@ struct RingArgs {
     uint64_t* status;
     uint32_t skip_origin;
     uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
+    uint32_t fetch_depth;                 // own rows through LDS: groups of LDS per wave-channel
 };
 
 struct Role {
@@ -249,12 +250,49 @@ struct FixedRole {
     static constexpr bool load = LOAD, recv = RECV, reduce = REDUCE, save = SAVE, send = SEND;
 };
 
+// ---- own rows through LDS ------------------------------------------------------
+// Vector-memory loads of one wavefront return in issue order, so a wave-channel
+// that fetches its own rows from HBM itself has every poll of staging (an L2
+// hit) queue behind the HBM fetch issued just before it: its step can never be
+// shorter than an HBM round trip, however far ahead it fetches.  With
+// MINT_FETCH_LDS a thread block carries one more wavefront, the *fetcher*: it
+// streams the own rows of the block's wave-channels from HBM, several groups
+// ahead, into a ring of LDS per wave-channel, and the wave-channels take them
+// from there (LDS operations count on another counter than vector memory).
+// Per wave-channel j of the block, in LDS:
+//   produced[j]   groups the fetcher has delivered     (fetcher writes)
+//   consumed[j]   groups the wave-channel has taken    (wave-channel writes)
+//   ring j        fetch_depth x U blocks of 1 KiB, arranged as ll_arrange leaves them
+#define MINT_LDS __attribute__((address_space(3)))
+constexpr uint32_t kLdsHeader = 64;       // the two counter arrays (8 wave-channels at most)
+struct LdsPort {
+    MINT_LDS uint8_t* ring;
+    MINT_LDS uint32_t* produced;
+    MINT_LDS uint32_t* consumed;
+    uint32_t depth;
+};
+__device__ __forceinline__ uint32_t lds_count(MINT_LDS uint32_t* p) {
+    return __builtin_amdgcn_readfirstlane(
+        __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+}
+__device__ __forceinline__ void lds_set(MINT_LDS uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ LdsPort lds_port(MINT_LDS uint8_t* base, int j, uint32_t depth, int U) {
+    LdsPort port;
+    port.produced = reinterpret_cast<MINT_LDS uint32_t*>(base) + j;
+    port.consumed = reinterpret_cast<MINT_LDS uint32_t*>(base) + 8 + j;
+    port.ring = base + kLdsHeader + (uint32_t)j * depth * (uint32_t)U * kBlockMsg;
+    port.depth = depth;
+    return port;
+}
+
 // The walk of one wave-channel along its rows, specialised by what its
 // position does (the flags are compile-time constants so that the loop of an
 // origin, an adder, a copier or a sink carries no tests for the other roles).
-template <int PROTO, int DT, int CPI, int U, typename RoleT>
+template <int PROTO, int DT, int CPI, int U, bool LDSF = false, typename RoleT>
 __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const int h, const int w,
-                                          const RoleT role) {
+                                          const RoleT role, const LdsPort port = LdsPort{}) {
     constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
     const LaneMap m;
     const uint64_t row_off = (uint64_t)p * a.row_stride;
@@ -292,7 +330,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
 #else
     constexpr bool timing = false;
 #endif
-    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0;
+    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0, t_lds = 0;
     const uint64_t t_begin = timing ? wall_clock64() : 0;
 
     // Group = U blocks of this wave-channel inside one step
@@ -331,6 +369,38 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         }
     };
 
+    // The own rows of the next whole group, taken out of LDS (LDSF): wait for
+    // the fetcher's count, read, hand the ring entry back.  LDS serves a
+    // wavefront's operations in order, so the fetcher that sees the new
+    // `consumed` knows the reads before it have been done.
+    uint32_t lds_taken = 0, lds_entry = 0;
+    auto lds_take = [&](u32x4 (&x)[U]) -> bool {
+        for (uint32_t spins = 0; lds_count(port.produced) <= lds_taken; ++spins) {
+            if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) return false;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        compiler_fence();
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            x[u] = *reinterpret_cast<MINT_LDS const u32x4*>(
+                port.ring + (lds_entry * (uint32_t)U + (uint32_t)u) * kBlockMsg + m.lane * 16u);
+        compiler_fence();
+        ++lds_taken;
+        lds_entry = lds_entry + 1 == port.depth ? 0 : lds_entry + 1;
+        lds_set(port.consumed, lds_taken);
+        return true;
+    };
+
+    // Own rows of the group being handled (v) and of the one fetched ahead
+    // (vnext).  The copy at the end of a group makes the group wait for the
+    // fetch it has issued after its polls, so a wave-channel never runs more
+    // than one fetch ahead of the ring.  That is on purpose.  Measured against
+    // two buffers that swap roles (loop unrolled by two, no wait at the end):
+    // the wave-channels then run ahead, arrive early at their polls and
+    // credit words, re-poll three times as often (0.19 - 0.78 re-polls per
+    // group instead of 0.01 - 0.26) and the launch takes 0.82 ms instead of
+    // 0.76: the L2 request rate, not a wavefront's latency, bounds the kernel,
+    // and every failed poll is eight more requests.
     u32x4 v[U], vnext[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
@@ -380,8 +450,18 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     r[u] = ld128<LDCP>(own, q.msg_off(geom, share_recv, u) + m.lane * 16u);
         }
         if (role.load) {
-            if (WHOLE) fetch_ahead(qn, vnext);
-            else load_own(q, v);
+            if (WHOLE && LDSF) {
+                const uint64_t t0 = timing ? wall_clock64() : 0;
+                if (!lds_take(v)) {
+                    report_timeout(a.status, p, h, w, s);
+                    return false;
+                }
+                if (timing) t_lds += wall_clock64() - t0;
+            } else if (WHOLE) {
+                fetch_ahead(qn, vnext);
+            } else {
+                load_own(q, v);
+            }
         }
         if (role.recv && PROTO == PROTO_LL128) {
             uint32_t pending = 0;
@@ -424,28 +504,30 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         for (int u = 0; u < U; ++u) {
             if (!(WHOLE || q.valid[u])) continue;
             const bool full = WHOLE || q.full[u];
-            if (role.load && PROTO == PROTO_LL128) v[u] = ll_arrange(v[u], full, m);
+            // (rows that came through LDS were arranged by the fetcher)
+            u32x4 x = v[u];
+            if (role.load && PROTO == PROTO_LL128 && !(WHOLE && LDSF)) x = ll_arrange(x, full, m);
             if (role.recv) {
                 if constexpr (DT != DT_BYTES) {
-                    v[u] = role.reduce ? ll_comp<DT>(v[u], r[u]) : r[u];
+                    x = role.reduce ? ll_comp<DT>(x, r[u]) : r[u];
                 } else {
-                    v[u] = r[u];
+                    x = r[u];
                 }
             }
             if (role.save) {
                 if (PROTO == PROTO_LL128) {
-                    ll_save_raw(out_row, row_bytes, q.g[u], full, m, v[u]);
+                    ll_save_raw(out_row, row_bytes, q.g[u], full, m, x);
                 } else {
                     const uint64_t off = (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u;
-                    if (full) st128_row(out_row + off, v[u]);
-                    else store_guarded(out_row, off, 16u, row_bytes, v[u]);
+                    if (full) st128_row(out_row + off, x);
+                    else store_guarded(out_row, off, 16u, row_bytes, x);
                 }
             }
             if (role.send) {
                 if (PROTO == PROTO_LL128)
-                    ll_send<STCP>(nxt, q.msg_off(geom, share_send, u), v[u], tag, m);
+                    ll_send<STCP>(nxt, q.msg_off(geom, share_send, u), x, tag, m);
                 else
-                    st128<STCP>(nxt, q.msg_off(geom, share_send, u) + m.lane * 16u, v[u]);
+                    st128<STCP>(nxt, q.msg_off(geom, share_send, u) + m.lane * 16u, x);
             }
         }
         if (q.last) {
@@ -466,7 +548,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 }
             }
         }
-        if (WHOLE) {
+        if (WHOLE && !LDSF) {
 #pragma unroll
             for (int u = 0; u < U; ++u) v[u] = vnext[u];
         }
@@ -631,7 +713,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     }
 
     // block numbers grow from group to group, so the whole groups come first
-    if (role.load && n < ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
+    if (!LDSF && role.load && n < ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
     while (n < ngroups && q.g[U - 1] < nfull)
         if (!run_group(std::true_type{})) return;
     while (n < ngroups)
@@ -645,14 +727,34 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         atomicAdd(st + 3, (unsigned long long)t_poll);
         atomicAdd(st + 4, (unsigned long long)(wall_clock64() - t_begin));
         atomicAdd(st + 5, 1ull);
+        atomicAdd(st + 6, (unsigned long long)t_lds);
     }
 }
 
-template <int PROTO, int DT, int CPI, int U>
-__global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
+// Which (pipeline, position, wave-channel) a wavefront serves.  `wpb` =
+// wave-channels per thread block, `wib` = this wavefront's index among them.
+struct Seat {
+    int p, h, gw, w;
+    bool ok;
+};
+__device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int wib) {
+    // Index of a wave-channel inside its group: it decides which blocks of
+    // a step, which staging bytes and which credit word the wave owns.  Under
+    // the local placement the blocks of one XCD are numbered consecutively, so
+    // that what an XCD touches (staging, rows) is contiguous in memory instead
+    // of 4 KiB out of every 32: that spreads it over all channels and sets of
+    // that XCD's L2.
+    if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
+        return (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
+    return gw * wpb + wib;
+}
+__device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib) {
+    Seat st;
+    st.ok = false;
+    st.p = st.h = st.gw = st.w = 0;
     const int npos = a.hops + 1;
     const int x = (int)blockIdx.x;
-    int c, h;
+    int c;
     if (a.placement == PLACE_LOCAL) {
         // Blocks are dealt round-robin over the XCDs, so every aligned group of
         // 8 consecutive blocks lands on 8 different XCDs - but not always block
@@ -668,43 +770,35 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
         const int xcd = xcc_id(), y = x / kXcds;
         if (xcd >= kXcds) {
             report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
-            return;
+            return st;
         }
-        h = y % npos;
+        st.h = y % npos;
         c = (y / npos) * kXcds + xcd;
     } else {
-        h = x % npos;
+        st.h = x % npos;
         c = x / npos;
     }
-    const int p = c / a.blocks_per_group;
-    // the wave index is the same in every lane: keep it (and all the index
-    // arithmetic that hangs off it) in scalar registers
-    const int wpb = (int)(blockDim.x >> 6);
-    const int gw = c % a.blocks_per_group;
-    const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
-    if (gw * wpb + wib >= a.waves) return;
-    // Index of this wave-channel inside its group: it decides which blocks of
-    // a step, which staging bytes and which credit word the wave owns.  Under
-    // the local placement the blocks of one XCD are numbered consecutively, so
-    // that what an XCD touches (staging, rows) is contiguous in memory instead
-    // of 4 KiB out of every 32: that spreads it over all channels and sets of
-    // that XCD's L2.
-    int w = gw * wpb + wib;
-    if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
-        w = (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
-    const Role role = role_of(a, p, h);
-    if (h == 0 && a.skip_origin) return;
+    st.p = c / a.blocks_per_group;
+    st.gw = c % a.blocks_per_group;
+    if (st.gw * wpb + wib >= a.waves) return st;
+    st.w = seat_wave(a, st.gw, wpb, wib);
+    st.ok = !(st.h == 0 && a.skip_origin);
+    return st;
+}
 
-    // one specialised walk per role
-    const int rk = role.rank, nx = role.next;
+// One specialised walk per role.
+template <int PROTO, int DT, int CPI, int U, bool LDSF>
+__device__ __forceinline__ void walk_as(const RingArgs& a, const Seat& st, const Role& role,
+                                        const LdsPort port = LdsPort{}) {
+    const int p = st.p, h = st.h, w = st.w, rk = role.rank, nx = role.next;
     if (!role.recv) {
-        ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, false, false, false, true>{rk, nx});
+        ring_walk<PROTO, DT, CPI, U, LDSF>(a, p, h, w, FixedRole<true, false, false, false, true>{rk, nx}, port);
     } else if (role.reduce) {
         if constexpr (DT != DT_BYTES) {
             if (role.save)
-                ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, true, true, true, true>{rk, nx});
+                ring_walk<PROTO, DT, CPI, U, LDSF>(a, p, h, w, FixedRole<true, true, true, true, true>{rk, nx}, port);
             else
-                ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<true, true, true, false, true>{rk, nx});
+                ring_walk<PROTO, DT, CPI, U, LDSF>(a, p, h, w, FixedRole<true, true, true, false, true>{rk, nx}, port);
         }
     } else if (role.send) {
         if (role.save)
@@ -714,6 +808,144 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     } else {
         ring_walk<PROTO, DT, CPI, U>(a, p, h, w, FixedRole<false, true, false, true, false>{rk, nx});
     }
+}
+
+template <int PROTO, int DT, int CPI, int U>
+__global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
+    // the wave index is the same in every lane: keep it (and all the index
+    // arithmetic that hangs off it) in scalar registers
+    const int wpb = (int)(blockDim.x >> 6);
+    const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
+    const Seat st = take_seat(a, wpb, wib);
+    if (!st.ok) return;
+    walk_as<PROTO, DT, CPI, U, false>(a, st, role_of(a, st.p, st.h));
+}
+
+// The fetcher wavefront of a thread block (MINT_FETCH_LDS): streams the own
+// rows of the block's WPB wave-channels into their LDS rings, R groups of
+// every wave-channel in flight in registers.  Wave-channel j of the block
+// handles, in group n, the blocks  step * step_blocks + (k0 + u) * W + w0 + j
+// (the walk of Group<U>); only whole groups come through LDS, the ragged end
+// of a row is loaded by the wave-channel itself.  Loads are issued
+// unconditionally (block numbers clamped into the row) so that the number of
+// loads in flight behind the one being delivered is the same on every path.
+template <int U, int WPB, int R>
+__device__ __forceinline__ void row_fetcher(const RingArgs& a, const Seat& st, const Role& role,
+                                            MINT_LDS uint8_t* lds) {
+    const LaneMap m;
+    uint64_t row_bytes;
+    uint32_t nblocks, nfull;
+    row_extent(a, st.p, kBlockRawLL, row_bytes, nblocks, nfull);
+    if (nfull == 0) return;
+    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) +
+                            (uint64_t)st.p * a.row_stride;
+    const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave, depth = a.fetch_depth;
+    const uint32_t ngroups = a.steps * (K / (uint32_t)U);
+    const uint32_t w0 = (uint32_t)seat_wave(a, st.gw, WPB, 0);
+    const int left = a.waves - st.gw * WPB;
+    const int nworkers = left < WPB ? left : WPB;
+    struct Cursor {
+        uint32_t step, k0;
+        __device__ __forceinline__ void advance(uint32_t K) {
+            k0 += (uint32_t)U;
+            if (k0 >= K) { k0 = 0; ++step; }
+        }
+    };
+    auto block_of = [&](const Cursor& c, int j, int u) {
+        return c.step * a.step_blocks + (c.k0 + (uint32_t)u) * W + w0 + (uint32_t)j;
+    };
+    u32x4 x[R][WPB][U];
+    Cursor ci{0u, 0u};
+    auto issue = [&](int r) {
+#pragma unroll
+        for (int j = 0; j < WPB; ++j)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                uint32_t g = block_of(ci, j, u);
+                g = g < nfull ? g : nfull - 1u;
+                x[r][j][u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
+            }
+        ci.advance(K);
+    };
+#pragma unroll
+    for (int r = 0; r < R; ++r) issue(r);
+    Cursor cd{0u, 0u};
+    uint32_t n = 0, entry = 0;
+    uint32_t freed[WPB];
+#pragma unroll
+    for (int j = 0; j < WPB; ++j) freed[j] = 0;
+#ifdef MINT_RING_STATS
+    const bool timing = a.stats != nullptr;
+#else
+    constexpr bool timing = false;
+#endif
+    uint64_t t_room = 0;
+    auto leave = [&]() {
+        if (timing && lane_id() == 0)
+            atomicAdd(reinterpret_cast<unsigned long long*>(a.stats) + 8 * st.h + 7,
+                      (unsigned long long)t_room);
+    };
+    for (;;) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            // block numbers grow with j: when wave-channel 0 has no whole group left, nobody has
+            if (n >= ngroups || block_of(cd, 0, U - 1) >= nfull) { leave(); return; }
+            const uint64_t t0 = timing ? wall_clock64() : 0;
+#pragma unroll
+            for (int j = 0; j < WPB; ++j) {
+                if (j >= nworkers || block_of(cd, j, U - 1) >= nfull) continue;
+                const LdsPort port = lds_port(lds, j, depth, U);
+                // room in the ring: the wave-channel has taken group n - depth
+                for (uint32_t spins = 0; n >= freed[j] + depth; ++spins) {
+                    freed[j] = lds_count(port.consumed);
+                    if (n < freed[j] + depth) break;
+                    if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
+                        report_timeout(a.status, st.p, st.h, (int)(w0 + (uint32_t)j), n);
+                        return;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                if (timing && j == WPB - 1) t_room += wall_clock64() - t0;
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    *reinterpret_cast<MINT_LDS u32x4*>(
+                        port.ring + (entry * (uint32_t)U + (uint32_t)u) * kBlockMsg + m.lane * 16u) =
+                        ll_arrange(x[r][j][u], true, m);
+            }
+            // LDS serves this wavefront's operations in order: the counts go
+            // out behind the data
+            compiler_fence();
+#pragma unroll
+            for (int j = 0; j < WPB; ++j)
+                if (j < nworkers && block_of(cd, j, U - 1) < nfull)
+                    lds_set(lds_port(lds, j, depth, U).produced, n + 1u);
+            compiler_fence();
+            issue(r);
+            cd.advance(K);
+            ++n;
+            entry = entry + 1 == depth ? 0 : entry + 1;
+        }
+    }
+}
+
+// The ring kernel with own rows through LDS: WPB wave-channels and one fetcher
+// per thread block.  LL128, reducing ops.
+template <int DT, int CPI, int U, int WPB, int R>
+__global__ void __launch_bounds__((WPB + 1) * 64) ring_kernel_lds(const RingArgs a) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    MINT_LDS uint8_t* lds = (MINT_LDS uint8_t*)lds_raw;
+    if (threadIdx.x < 16) reinterpret_cast<MINT_LDS uint32_t*>(lds)[threadIdx.x] = 0u;
+    __syncthreads();
+    const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
+    const bool fetcher = wib == WPB;
+    const Seat st = take_seat(a, WPB, fetcher ? 0 : wib);
+    if (!st.ok) return;
+    const Role role = role_of(a, st.p, st.h);
+    if (fetcher) {
+        if (role.load) row_fetcher<U, WPB, R>(a, st, role, lds);
+        return;
+    }
+    walk_as<PROTO_LL128, DT, CPI, U, true>(a, st, role, lds_port(lds, wib, a.fetch_depth, U));
 }
 
 }  // namespace mint

@@ -11,37 +11,83 @@
 namespace mint {
 namespace {
 
+// Thread blocks of `threads` threads (and `lds_bytes` of LDS) that a CU holds
+// at once.  Every wavefront of a ring launch polls words other wavefronts
+// write, so the whole grid has to be resident.  The occupancy query is asked
+// twice: for the block size, and for blocks of one wavefront, which tells how
+// many wavefronts of this kernel a CU takes.  Of those at most 6 per SIMD are
+// counted.  Measured: where the query says 7 (the kernels need 98 - 106
+// scalar registers), a grid of 6 blocks of 4 wavefronts per CU runs in one go
+// and one of 7 takes a third longer - the query does not see the scalar
+// registers the platform sets aside per wavefront for its trap handler (a
+// build squeezed into 16 fewer registers moved the step by exactly one
+// wavefront per SIMD).
+template <typename Kernel>
+int resident_blocks_per_cu(Kernel kernel, int threads, size_t lds_bytes) {
+    int per_cu = 0, waves_per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, lds_bytes) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&waves_per_cu, kernel, 64, 0) != hipSuccess)
+        return -1;
+    if (waves_per_cu > 24) waves_per_cu = 24;
+    const int by_waves = waves_per_cu / (threads / 64);
+    if (by_waves < per_cu) per_cu = by_waves;
+    return per_cu < 1 ? 1 : per_cu;
+}
+
+// Own rows through LDS (reducing element types only): WPB wave-channels and
+// one fetcher wavefront per thread block, R groups in flight per wave-channel.
+template <int DT, int CP>
+int launch_ring_lds(const Plan& plan, hipStream_t stream) {
+    if constexpr (DT == DT_BYTES) {
+        return MINT_ERR_ARG;
+    } else {
+        const int wpb = plan.threads / 64;
+        void (*kernel)(const RingArgs) = nullptr;
+        if (wpb == 4)
+            kernel = plan.unroll == 2 ? ring_kernel_lds<DT, CP, 2, 4, 2> : ring_kernel_lds<DT, CP, 1, 4, 3>;
+        else
+            kernel = plan.unroll == 2 ? ring_kernel_lds<DT, CP, 2, 7, 1> : ring_kernel_lds<DT, CP, 1, 7, 2>;
+        const int threads = plan.threads + 64;
+        const size_t lds_bytes = kLdsHeader + (size_t)wpb * plan.args.fetch_depth *
+                                                  (size_t)plan.unroll * kBlockMsg;
+        static std::atomic<int> cached[2][2] = {};       // [wpb == 7][unroll == 2]
+        static std::atomic<int> cus{0};
+        std::atomic<int>& memo = cached[wpb == 7][plan.unroll == 2];
+        int per_cu = memo.load(std::memory_order_relaxed);
+        if (per_cu == 0) {
+            per_cu = resident_blocks_per_cu(kernel, threads, lds_bytes);
+            if (per_cu < 0) return MINT_ERR_HIP;
+            memo.store(per_cu, std::memory_order_relaxed);
+        }
+        int ncu = cus.load(std::memory_order_relaxed);
+        if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
+        if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)threads), lds_bytes,
+                           stream, plan.args);
+        return launch_status();
+    }
+}
+
 template <int PROTO, int DT, int CP>
 int launch_ring_u(const Plan& plan, hipStream_t stream) {
+    if (plan.lds) return launch_ring_lds<DT, CP>(plan, stream);
     void (*kernel)(const RingArgs) = nullptr;
     switch (plan.unroll) {
         case 4: kernel = ring_kernel<PROTO, DT, CP, 4>; break;
         case 2: kernel = ring_kernel<PROTO, DT, CP, 2>; break;
         default: kernel = ring_kernel<PROTO, DT, CP, 1>; break;
     }
-    // Every wavefront of the launch polls words other wavefronts write, so
-    // the whole grid has to be resident at once.  The occupancy of a kernel
-    // at a block size does not change: ask once (per block size) and keep it.
-    // (these statics are per template instantiation, i.e. per kernel family)
+    // The occupancy of a kernel at a block size does not change: ask once
+    // (per block size) and keep it.  (These statics are per template
+    // instantiation, i.e. per kernel family.)
     static std::atomic<int> cached[3][9] = {};       // [unroll][threads / 64]
     static std::atomic<int> cus{0};
     std::atomic<int>& memo = cached[plan.unroll == 4 ? 2 : (plan.unroll == 2 ? 1 : 0)]
                                    [plan.threads / 64];
     int per_cu = memo.load(std::memory_order_relaxed);
     if (per_cu == 0) {
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, plan.threads, 0) !=
-            hipSuccess)
-            return MINT_ERR_HIP;
-        // Count one wavefront per SIMD less than the query allows.  Measured:
-        // at 4 waves per block the query says 7 blocks per CU, yet from 6
-        // blocks per CU on the grid is no longer dealt out in one go and a
-        // launch takes a third longer (the query does not see the scalar
-        // registers the platform sets aside per wave for its trap handler;
-        // a build squeezed into 16 fewer registers moved the step by exactly
-        // one wave per SIMD).
-        const int waves_per_block = plan.threads / 64;
-        per_cu = (per_cu * waves_per_block - 4) / waves_per_block;
-        if (per_cu < 1) per_cu = 1;
+        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
+        if (per_cu < 0) return MINT_ERR_HIP;
         memo.store(per_cu, std::memory_order_relaxed);
     }
     int ncu = cus.load(std::memory_order_relaxed);

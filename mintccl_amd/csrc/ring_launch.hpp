@@ -15,6 +15,8 @@ struct Plan {
     int blocks, threads, unroll;
     size_t staging_need;      // bytes of staging per rank: slots + credit words
     bool empty;
+    bool lds;                 // own rows through LDS: `threads` counts the wave-channels'
+                              // threads only, the launch adds the fetcher wavefront
 };
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? MINT_OK : MINT_ERR_HIP; }

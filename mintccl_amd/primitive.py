@@ -43,6 +43,22 @@ def read_xor(src: torch.Tensor, out: torch.Tensor | None = None, blocks: int = 0
     return out
 
 
+def step_mix(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int, iters: int,
+             what: int = 7, sink: torch.Tensor | None = None) -> None:
+    """The memory accesses of ``waves`` x ``iters`` ring steps with no ring around
+    them (``what``: 1 own-row loads from ``rows``, 2 loads from ``staging``,
+    4 stores into ``staging``): the yardstick for what the device can do with
+    the ring kernels' mix of accesses."""
+    ref = rows if rows is not None else staging
+    if sink is None and not what & 4:
+        sink = torch.zeros(1, dtype=torch.int32, device=ref.device)
+    nb = lambda t: 0 if t is None else t.numel() * t.element_size()
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(ref.device):
+        _lib.check(_lib.lib().mint_step_mix(ptr(rows), nb(rows), ptr(staging), nb(staging), waves,
+                                            iters, what, ptr(sink), _stream(ref)), "mint_step_mix")
+
+
 def Sum(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """Elementwise ``rn(a + b)``, one rounding, by the ring kernels' own adder."""
     if a.dtype not in DTYPE_CODE or a.dtype != b.dtype or a.numel() != b.numel():

@@ -48,6 +48,7 @@ def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None,
         route = find_route(s["rank"], r["rank"], topo)
     if not route or route[0] != s["rank"] or route[-1] != r["rank"]:
         raise ValueError(f"no route {s['rank']} -> {r['rank']}")
+    comm.last_route = list(route)
     d = comm.make_op(_lib.OP_SENDRECV, _lib.BYTES, s["count"], {s["rank"]: s["data_ptr"]},
                      {r["rank"]: r["data_ptr"]}, route, route_len=len(route))
     if full_size_staging:

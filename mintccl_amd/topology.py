@@ -5,10 +5,16 @@ same two entry points, built to their stated intent - ``find_ring`` returns a
 Hamiltonian cycle through node 0 that maximises the bottleneck bandwidth,
 ``find_route`` the widest path (direct link first, or the shortest path on
 request).  The virtual ranks of one GPU form a uniform complete graph, for
-which the ring is ``[0, 1, ..., N-1, 0]``.  The bandwidth probe of
-``topology.py:96-150`` needs several GPUs and is not part of this build;
-``get_topology`` returns the uniform graph or loads a ``topo.json`` of the
-reference's format ``{src: [[dst, GB/s], ...]}``.
+which the ring is ``[0, 1, ..., N-1, 0]``.
+
+``get_topology`` loads a ``topo.json`` of the reference's format
+(``topology.py:128-150``: ``{"src": [[dst, GB/s], ...], ...}``, keys turned
+into strings by ``json.dump``), or returns the uniform graph; ``save_topology``
+writes that format; ``probe_topology`` is the reference's measurement pass
+(``get_p2p_speed`` for every pair, ``topology.py:96-126,135-148``) run between
+the buffers of virtual ranks, where a "link" is a copy inside one GPU's HBM
+(the peer-to-peer copies between GPUs that the reference times need more than
+one GPU).
 """
 from __future__ import annotations
 
@@ -37,6 +43,57 @@ def get_topology(topo: str = "topo.json", world_size: int | None = None) -> Topo
         from .common import get_comm
         world_size = get_comm().world_size
     return uniform_topology(world_size)
+
+
+def save_topology(topo: Topology, path: str = "topo.json") -> None:
+    """Write ``topo`` the way the reference persists it (``topology.py:148-149``):
+    one entry per source, its links as ``[dst, bandwidth]`` pairs, widest
+    first (the reference's own ``sorted(items, reverse=True)`` orders by
+    destination id; the stated intent - "sorted", widest first - is what is
+    written, and readers accept any order)."""
+    doc = {str(src): [[int(d), float(bw)] for d, bw in sorted(links, key=lambda e: (-e[1], e[0]))]
+           for src, links in sorted(topo.items())}
+    with open(path, "w") as f:
+        json.dump(doc, f)
+
+
+def get_p2p_speed(src: int, dst: int, size: int = 33554432, comm=None) -> float:
+    """GB/s of a ``size``-byte copy from virtual rank ``src`` to virtual rank
+    ``dst`` (``topology.py:96-126``; there a ``cudaMemcpyPeerAsync`` between two
+    GPUs, here the library's own copy kernel between two buffers of one GPU),
+    timed with events on the current stream."""
+    import torch
+
+    from . import primitive
+    from .common import get_comm
+    comm = comm if comm is not None else get_comm()
+    a = torch.empty(size, dtype=torch.uint8, device=comm.device)
+    b = torch.empty(size, dtype=torch.uint8, device=comm.device)
+    primitive.copy128(a, b)                                  # first touch
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    primitive.copy128(a, b)
+    stop.record()
+    torch.cuda.synchronize(comm.device)
+    return size / (start.elapsed_time(stop) / 1e3) / 1e9
+
+
+def probe_topology(world_size: int | None = None, path: str | None = None, comm=None) -> Topology:
+    """Measure every pair once, both directions get the same figure
+    (``topology.py:135-148``), and persist the result if ``path`` is given."""
+    from .common import get_comm
+    comm = comm if comm is not None else get_comm()
+    world_size = world_size if world_size is not None else comm.world_size
+    topo: Topology = {s: [] for s in range(world_size)}
+    for s in range(world_size):
+        for d in range(s + 1, world_size):
+            bw = get_p2p_speed(s, d, comm=comm)
+            topo[s].append((d, bw))
+            topo[d].append((s, bw))
+    topo = {s: sorted(links, key=lambda e: (-e[1], e[0])) for s, links in topo.items()}
+    if path is not None:
+        save_topology(topo, path)
+    return topo
 
 
 def find_route(src: int, dst: int, topo: Topology | None = None,

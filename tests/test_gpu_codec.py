@@ -169,3 +169,32 @@ def test_alignment_is_rejected_not_faulted(lib, dev):
     assert lib.mint_ll128_pack(p + 8, p + 2048, 64, 1, 1, 0, 0) == _lib.ERR_ALIGN
     assert lib.mint_ll128_pack(p, p + 2048, 64, 1, 1, 5, 0) == _lib.ERR_ARG
     assert lib.mint_elementwise_sum(p, p + 4, p + 2048, 8, 0, 0) == _lib.ERR_ALIGN
+
+
+def test_step_mix_moves_what_it_says(dev):
+    """The access-mix yardstick: with own-row loads and stores selected, the
+    slot a wave stores into in its last step holds that step's own block in
+    the lane order of the raw side (lane l, l % 4 != 3, carries the aligned
+    16-byte vector l - l // 4 of the block)."""
+    from mintccl_amd import primitive
+    waves, iters = 37, 5
+    # f16 values in [1, 2): the store carries own + 0, which keeps such bits as they are
+    rows = (torch.rand(waves * iters * 480, device=dev) + 1).to(torch.float16).view(torch.uint8)
+    staging = torch.zeros(waves * 2048, dtype=torch.uint8, device=dev)
+    primitive.step_mix(rows, staging, waves, iters, what=1 | 4)
+    torch.cuda.synchronize()
+    r, s = rows.cpu().numpy(), staging.cpu().numpy()
+    for w in (0, 1, 17, waves - 1):
+        block = r[((iters - 1) * waves + w) * 960:][:960]
+        slot = s[w * 2048 + (iters & 1) * 1024:][:1024]
+        for lane in range(64):
+            if lane % 4 != 3:
+                vec = lane - lane // 4
+                assert (slot[lane * 16: lane * 16 + 16] == block[vec * 16: vec * 16 + 16]).all()
+    # all three at once only has to run; loads alone leave staging as it is
+    before = staging.clone()
+    primitive.step_mix(rows, staging, waves, iters, what=1 | 2)
+    torch.cuda.synchronize()
+    assert torch.equal(staging, before)
+    primitive.step_mix(rows, staging, waves, iters, what=7)
+    torch.cuda.synchronize()

@@ -100,6 +100,48 @@ def test_reducescatter_dtypes_protocols_placements(dev, dt, proto, place, cp):
     assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], dt))
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("threads", [256, 448])
+@pytest.mark.parametrize("world,n", [(8, 100003), (8, 480 * 64 * 3), (3, 4099), (5, 7)])
+def test_reducescatter_with_own_rows_through_lds(dev, dt, threads, world, n):
+    """MINT_FETCH_LDS: one more wavefront per thread block streams the own rows
+    into LDS and the wave-channels take them from there.  Same bits as the
+    oracle, for thread blocks of 4 and of 7 wave-channels, the tuned geometry
+    and small ones with one and with two blocks per wave-channel and step."""
+    from mintccl_amd import _lib
+    host = rank_rows(world, n, dt, seed0=n)
+    want = ring.reducescatter([as_bytes(h) for h in host], dt)
+    wpb = threads // 64
+    for kw in (dict(), dict(buff_size_=world * 2 * wpb * 2048, nslots=2, waves_per_rank=2 * wpb * world),
+               dict(buff_size_=world * 4 * wpb * 2048, nslots=2, waves_per_rank=2 * wpb * world)):
+        bufs = [h.to(dev) for h in host]
+        comm = make_comm(world, row_fetch=_lib.FETCH_LDS, threads_per_block=threads, **kw)
+        run_reducescatter(comm, bufs)
+        assert same(bufs, want), kw
+
+
+@pytest.mark.parametrize("world", [2, 8])
+def test_reduce_and_allreduce_with_own_rows_through_lds(dev, world):
+    from mintccl_amd import _lib
+    from mintccl_amd.allreduce import allreduce
+    n = 70001
+    host = [normal(n, 50 + r) for r in range(world)]
+    raw = [as_bytes(h) for h in host]
+    comm = make_comm(world, row_fetch=_lib.FETCH_LDS)
+    bufs = [h.to(dev) for h in host]
+    run_reduce(comm, bufs, world - 1)
+    assert same(bufs, ring.reduce(raw, world - 1, "f16"))
+    for fused in (False, True):
+        bufs = [h.to(dev) for h in host]
+        comm.run(lambda r: allreduce(bufs[r], comm, fused=fused))
+        comm.check()
+        assert same(bufs, ring.allreduce(raw, "f16"))
+    # the copying collectives have no such kernel: the option is ignored
+    bufs = [h.to(dev) for h in host]
+    run_broadcast(comm, bufs, 0)
+    assert same(bufs, ring.broadcast(raw, 0))
+
+
 def test_reducescatter_special_values(dev):
     # overflow to inf, inf - inf, subnormals, signed zeros ride the ring unharmed
     world, n = 4, 960
@@ -277,6 +319,46 @@ def test_permuted_ring(dev):
     bufs2 = [h.to(dev) for h in host2]
     run_reduce(comm, bufs2, 1)
     assert same(bufs2, ring.reduce([as_bytes(h) for h in host2], 1, "f16", ring_))
+
+
+def test_topology_file_drives_ring_and_route_end_to_end(dev, tmp_path):
+    """A non-uniform ``topo.json`` (the reference's file format), written with
+    ``save_topology`` and loaded with ``get_topology``: the collectives run
+    round the ring it implies, and the deferred send / recv takes the widest
+    route - three hops, 0 -> 2 -> 1 -> 3 (bottleneck 47.5 against 24 via rank 1
+    alone and 23 via rank 2 alone; ranks 0 and 3 have no direct link)."""
+    from mintccl_amd import sendrecv_buffer
+    from mintccl_amd.topology import find_ring, find_route, get_topology, save_topology
+    world = 4
+    links = {(0, 2): 48.0, (2, 1): 47.5, (1, 3): 48.5, (0, 1): 24.0, (2, 3): 23.0}
+    topo = {i: [] for i in range(world)}
+    for (a, b), bw in links.items():
+        topo[a].append((b, bw))
+        topo[b].append((a, bw))
+    path = str(tmp_path / "topo.json")
+    save_topology(topo, path)
+    comm = make_comm(world)
+    comm.topology = get_topology(path)
+    ring_ = find_ring(comm.topology)
+    assert ring_ in ([0, 1, 3, 2, 0], [0, 2, 3, 1, 0])          # the two cycles there are
+    assert find_route(0, 3, comm.topology) == [0, 2, 1, 3]
+    host = rank_rows(world, 20008, "f16")
+    bufs = [h.to(dev) for h in host]
+    run_reducescatter(comm, bufs)
+    assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16", ring_))
+    bufs = [h.to(dev) for h in host]
+    run_allgather(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    src = normal(300007, 9).to(dev)
+    dst = torch.zeros_like(src)
+    with comm.rank(0):
+        sendrecv_buffer.send(src, 3, comm)
+    with comm.rank(3):
+        sendrecv_buffer.recv(dst, 0, comm)
+    sendrecv_buffer.sync(comm)                               # route from the topology
+    comm.check()
+    assert torch.equal(dst.view(torch.int16), src.view(torch.int16))
+    assert comm.last_route == [0, 2, 1, 3]
 
 
 def test_many_launches_reuse_staging_without_clearing(dev):
@@ -463,8 +545,11 @@ def test_one_flag_per_128_byte_line_is_not_enough(lib, dev):
     pairs, iters = 2048, 20000
     checked, torn, polls, timeouts, first_half = run_probe(lib, dev, pairs, iters, 0, 0, 0)[:5]
     assert timeouts == 0 and checked == pairs * iters * 8
-    assert torn == first_half
     print(f"lines checked {checked}, torn {torn} (first sector stale: {first_half})")
+    # How often a line tears depends on the machine's load and may be zero in
+    # a short run; what is pinned is the shape of a tear when there is one.
+    if torn:
+        assert torn == first_half
 
 
 # ---- the benchmark configurations at their full sizes -----------------------
@@ -481,17 +566,23 @@ def test_config3_broadcast_64mib_8_ranks(dev):
 
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 def test_config4_reducescatter_and_reduce_32m_elements(dev, dt):
-    # 32 Mi elements per rank, seed 3000 + rank, 1 MiB slots.  Full-size check
-    # against the device adder folded in ring order (itself checked against the
-    # oracle above), plus the oracle on a slice of every chunk.
+    # 32 Mi elements per rank, seed 3000 + rank, 1 MiB slots.  Every owner row,
+    # whole, against the oracle's fold on the host (the arithmetic and the
+    # order at full size); rows a rank does not own must come back untouched.
+    # The device adder folded in ring order is kept beside it as a second,
+    # independent route to the same bits.
     from mintccl_amd import primitive
     world, n_total = 8, 33554432
     n = n_total // world
-    bufs = [normal(n_total, 3000 + r, TORCH_DT[dt]).reshape(world, n).to(dev) for r in range(world)]
+    host = [normal(n_total, 3000 + r, TORCH_DT[dt]).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
     orig = [b.clone() for b in bufs]
     comm = make_comm(world, buff_size_=8 << 20, nslots=8, waves_per_rank=256)
     run_reducescatter(comm, bufs)
     for c in range(world):
+        want = ring.fold([as_bytes(host[r][c]) for r in range(world)],
+                         ring.fold_order(ring.identity_ring(world), c), dt)
+        assert np.array_equal(as_bytes(bufs[c][c]), want), c
         acc = orig[c][c].clone()
         for k in range(1, world):
             acc = primitive.Sum(orig[(c + k) % world][c].contiguous(), acc)
@@ -499,19 +590,18 @@ def test_config4_reducescatter_and_reduce_32m_elements(dev, dt):
         for r in range(world):
             if r != c:
                 assert torch.equal(bufs[r][c], orig[r][c])
-        sl = slice(n - 4099, n)
-        want = ring.fold([as_bytes(orig[r][c, sl]) for r in range(world)],
-                         ring.fold_order(ring.identity_ring(world), c), dt)
-        assert np.array_equal(as_bytes(bufs[c][c, sl]), want)
     flat = [o.reshape(-1).clone() for o in orig]
     run_reduce(comm, flat, 0)
-    acc = orig[0].reshape(-1).clone()
-    for k in range(1, world):
-        acc = primitive.Sum(orig[k].reshape(-1), acc)
-    assert torch.equal(flat[0].view(torch.uint8), acc.view(torch.uint8))
+    want = ring.fold([as_bytes(h) for h in host], ring.fold_order(ring.identity_ring(world), 0), dt)
+    assert np.array_equal(as_bytes(flat[0]), want)
+    for r in range(1, world):
+        assert torch.equal(flat[r], orig[r].reshape(-1))
 
 
 def test_headline_reducescatter_256mib_fp16(dev):
+    """8 ranks x 256 MiB fp16 with the library's default geometry (the one
+    bench.py times): every owner row, all 32 MiB of it, against the oracle's
+    fold computed on the host, and every other row untouched."""
     from mintccl_amd import primitive
     world, n_total = 8, 134217728
     n = n_total // world
@@ -521,10 +611,17 @@ def test_headline_reducescatter_256mib_fp16(dev):
     comm = make_comm(world)
     run_reducescatter(comm, bufs)
     for c in range(world):
+        rows = [as_bytes(orig[r][c]) for r in range(world)]
+        want = ring.fold(rows, ring.fold_order(ring.identity_ring(world), c), "f16")
+        assert np.array_equal(as_bytes(bufs[c][c]), want), c
+        del rows, want
         acc = orig[c][c].clone()
         for k in range(1, world):
             acc = primitive.Sum(orig[(c + k) % world][c].contiguous(), acc)
         assert torch.equal(bufs[c][c].view(torch.int16), acc.view(torch.int16))
+        for r in range(world):
+            if r != c:
+                assert torch.equal(bufs[r][c].view(torch.int16), orig[r][c].view(torch.int16)), (r, c)
 
 
 def test_empty_buffers_are_a_no_op(dev):

@@ -82,3 +82,49 @@ def test_find_route_is_widest(seed):
 def test_find_plan():
     assert topology.find_plan([0, 2, 1, 3, 0], 1) == (2, 3)
     assert topology.find_plan([0, 1, 0], 0) == (1, 1)
+
+
+def test_topo_json_round_trip_in_the_reference_format(tmp_path):
+    """``topo.json`` as the reference writes it (``topology.py:128-150``): a
+    dict keyed by the source rank - a string once it has been through JSON -
+    of ``[dst, GB/s]`` pairs.  What ``save_topology`` writes is that, and
+    ``get_topology`` reads it back unchanged."""
+    import json
+    rng = random.Random(7)
+    topo = random_topology(6, rng, p=0.7)
+    topo = {s: sorted(links, key=lambda e: (-e[1], e[0])) for s, links in topo.items()}
+    path = tmp_path / "topo.json"
+    topology.save_topology(topo, str(path))
+    doc = json.load(open(path))
+    assert sorted(doc) == [str(s) for s in range(6)]
+    for s, links in doc.items():
+        assert all(isinstance(d, int) and isinstance(bw, float) for d, bw in links)
+        assert [bw for _, bw in links] == sorted((bw for _, bw in links), reverse=True)
+    assert topology.get_topology(str(path)) == topo
+    assert topology.find_ring(topology.get_topology(str(path))) == topology.find_ring(topo)
+
+
+def test_topo_json_written_the_reference_way_is_read(tmp_path):
+    # the reference sorts every list with sorted(items, reverse=True): by
+    # destination id, descending (topology.py:148), and dumps int keys
+    import json
+    raw = {0: [(1, 48.2), (2, 23.9), (3, 24.1)], 1: [(0, 48.2), (2, 24.0), (3, 47.9)],
+           2: [(0, 23.9), (1, 24.0), (3, 48.0)], 3: [(0, 24.1), (1, 47.9), (2, 48.0)]}
+    as_reference = {src: sorted(items, reverse=True) for src, items in raw.items()}
+    path = tmp_path / "topo.json"
+    json.dump(as_reference, open(path, "w"))
+    topo = topology.get_topology(str(path))
+    assert set(topo) == {0, 1, 2, 3}
+    assert topo[0] == [(1, 48.2), (3, 24.1), (2, 23.9)]        # widest first
+    # the ring through the three wide links and one narrow one: 0-1-3-2-0 (bottleneck 23.9)
+    # against 0-1-2-3-0 (24.0) and 0-2-1-3-0 (23.9): the best bottleneck is 24.0
+    ring = topology.find_ring(topo)
+    assert otopo.ring_bandwidth(topo, ring) == otopo.best_ring_bandwidth(topo) == 24.0
+    assert topology.find_route(0, 2, topo) == [0, 2]                   # a direct link wins
+    missing = {s: [(d, bw) for d, bw in links if {s, d} != {0, 2}] for s, links in topo.items()}
+    assert topology.find_route(0, 2, missing) == [0, 1, 3, 2]          # widest: min(48.2, 47.9, 48.0)
+
+
+def test_get_topology_without_a_file_is_uniform(tmp_path):
+    topo = topology.get_topology(str(tmp_path / "absent.json"), world_size=4)
+    assert topo == topology.uniform_topology(4)

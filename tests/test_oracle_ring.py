@@ -217,3 +217,23 @@ def test_allreduce_chunks_and_order():
     padded = [np.concatenate([x, np.zeros(world * row - x.size, np.uint8)]) for x in xs]
     want = ring.allgather(ring.reducescatter(padded, "f16"))[0][:2 * n]
     assert all((o == want).all() for o in ring.allreduce(xs, "f16"))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("world,n", [(8, 1000), (3, 481), (4, 7), (2, 960)])
+def test_torch_cpu_walk_equals_the_numpy_walk(dt, world, n):
+    """The PyTorch-CPU walk that bench.py times as the CPU baseline gives the
+    bits of the numpy restatement (which the tests above pin), through the
+    wire format, for a permuted ring as well."""
+    import torch
+    from oracle import torch_ring
+    g = torch.Generator().manual_seed(world * 1000 + n)
+    bufs = [torch.randn(world, n, generator=g).to(torch_ring.TORCH_DT[dt]) for _ in range(world)]
+    raw = [b.view(torch.uint8).numpy().reshape(-1) for b in bufs]
+    rings = [None, list(reversed(range(world))) + [world - 1]]
+    for rg in rings:
+        got = torch_ring.reducescatter_wire(bufs, dt, ring=rg, flag_base=(1 << 32) - 5)
+        want = ring.reducescatter_wire(raw, dt, ring=rg, flag_base=(1 << 32) - 5)
+        assert ring.reducescatter(raw, dt, ring=rg)[0].tobytes() == want[0].tobytes()
+        for r in range(world):
+            assert np.array_equal(got[r].view(torch.uint8).numpy().reshape(-1), want[r]), r
