@@ -57,8 +57,13 @@ typedef enum {
     MINT_OP_REDUCE = 2,        /* 5_reduce.py:36-95 */
     MINT_OP_ALLGATHER = 3,     /* 6_allgather.py:79-138 (spatial variant) */
     MINT_OP_REDUCESCATTER = 4, /* 7_reducescatter.py:13-79 */
-    MINT_OP_ALLREDUCE = 5      /* the reference's planned 8_allreduce (README.md:23):
+    MINT_OP_ALLREDUCE = 5,     /* the reference's planned 8_allreduce (README.md:23):
                                   reducescatter and allgather in one pass round the ring */
+    MINT_OP_ALLTOALL = 6       /* the reference's planned 9_alltoall (README.md:24,50):
+                                  row d of rank s goes into row s of rank d, every
+                                  row straight to its destination through the
+                                  destination's staging (input[] and output[] must
+                                  not overlap) */
 } mint_op;
 typedef enum {
     MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
@@ -112,11 +117,13 @@ typedef struct {
                               words sit behind the slots, outside a buffer
                               that only holds nslots * slot_bytes) */
     uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE: bytes of the
-                              buffer; ALLGATHER/REDUCESCATTER: bytes of one row */
-    uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER: bytes between rows */
+                              buffer; ALLGATHER/REDUCESCATTER/ALLTOALL: bytes of
+                              one row */
+    uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER/ALLTOALL: bytes between rows */
     uint32_t slot_bytes;   /* staging bytes of one step over all pipelines;
                               multiple of 1024, >= 1024 per pipeline (per
-                              pipeline and phase for ALLREDUCE, which has 2) */
+                              pipeline and phase for ALLREDUCE, which has 2;
+                              per source rank for ALLTOALL) */
     uint32_t nslots;       /* slots in the circular staging buffer */
     uint32_t waves_per_channel_group; /* wave-channels per (pipeline, hop) */
     uint32_t threads_per_block;       /* multiple of 64 */

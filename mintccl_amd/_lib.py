@@ -27,7 +27,8 @@ MAX_EPOCH = 4095          # sector tags carry a 12-bit launch epoch
 LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
 F16, BF16, F32, BYTES = 0, 1, 2, 3
 PROTO_LL128, PROTO_SIMPLE = 0, 1
-OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER, OP_ALLREDUCE = range(6)
+(OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER, OP_ALLREDUCE,
+ OP_ALLTOALL) = range(7)
 PLACE_SPREAD, PLACE_LOCAL = 0, 1
 FETCH_INLINE, FETCH_LDS = 0, 1
 

@@ -141,6 +141,13 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
     geometry for one collective: the wavefront budget spread over the
     (pipeline, hop) groups, one 1 KiB block per wave-channel per step, whole
     thread blocks, and a channel count the 8 XCDs divide."""
+    if op == _lib.OP_ALLTOALL:
+        # world x world pipelines of two positions; a rank's slot has one share
+        # per source rank
+        total = TUNED_TOTAL_WAVES_MULTI
+        wpb = max(1, threads_per_block // 64)
+        waves = max(wpb, total // (2 * world * world) // wpb * wpb)
+        return world * waves * 1024, min(max_nslots, TUNED_NSLOTS_MULTI), waves
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
     real_pipes = pipes
     if op == _lib.OP_ALLREDUCE:
@@ -347,7 +354,7 @@ class VirtualComm:
         # credit words at a fixed place, whatever slot geometry a launch uses
         d.credit_offset = self.buff_size
         pipes = self.world_size if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER,
-                                          _lib.OP_ALLREDUCE) else 1
+                                          _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL) else 1
         if op == _lib.OP_ALLREDUCE:
             pipes *= 2            # a slot is shared by (pipeline, phase): two phases
         if self.auto_geometry:
@@ -362,8 +369,11 @@ class VirtualComm:
             if self.slot_bytes % 1024 or step_blocks == 0:
                 raise ValueError(
                     "slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
+            # (an alltoall has twice `pipes` groups of wave-channels per rank: it
+            # sends `world` rows and receives `world` rows)
+            groups = 2 * pipes if op == _lib.OP_ALLTOALL else pipes
             d.waves_per_channel_group = _largest_divisor_at_most(
-                step_blocks, max(1, self.waves_per_rank // pipes))
+                step_blocks, max(1, self.waves_per_rank // groups))
         d.threads_per_block = self.threads_per_block
         d.placement, d.cache_policy = self.placement, self.cache_policy
         d.row_fetch = self.row_fetch
@@ -372,6 +382,8 @@ class VirtualComm:
             # does not divide, this launch runs spread with agent-scope staging
             wpb = max(1, min(self.threads_per_block // 64, d.waves_per_channel_group))
             real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
+            if op == _lib.OP_ALLTOALL:
+                real_pipes = self.world_size * self.world_size
             channels = real_pipes * -(-d.waves_per_channel_group // wpb)
             if channels % 8:
                 d.placement = _lib.PLACE_SPREAD

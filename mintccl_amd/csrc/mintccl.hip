@@ -41,7 +41,7 @@ bool reducing(int op) {
 int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
               const mint_ring_debug* dbg = nullptr) {
     if (!op || !plan) return MINT_ERR_ARG;
-    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLREDUCE) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLTOALL) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
@@ -67,9 +67,14 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     a.op = op->op;
     a.world = op->world;
     const bool allreduce = op->op == MINT_OP_ALLREDUCE;
-    const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER || allreduce;
-    a.pipes = rowwise ? op->world : 1;
+    const bool alltoall = op->op == MINT_OP_ALLTOALL;
+    const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER ||
+                         allreduce || alltoall;
+    a.pipes = alltoall ? op->world * op->world : (rowwise ? op->world : 1);
     a.phases = allreduce ? 2 : 1;
+    // a rank receives from every pipeline that passes through it: one share of
+    // its slots per pipeline and phase; in an alltoall, one per source rank
+    a.shares = alltoall ? op->world : a.pipes * a.phases;
 
     // ring / route
     bool seen[MINT_MAX_RANKS] = {};
@@ -78,6 +83,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         a.cyc_len = op->route_len;
     } else {
         a.cyc_len = op->world;
+        // (an alltoall sends every row straight to its destination: the ring
+        // is not walked, but it still has to be one)
         if (op->ring[op->world] != op->ring[0]) return MINT_ERR_ARG;
     }
     for (int i = 0; i < a.cyc_len; ++i) {
@@ -99,6 +106,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
             a.start[0] = (uint8_t)index_of(op->root);
             break;
         }
+        case MINT_OP_ALLTOALL: a.hops = 1; break;
         default:
             a.hops = op->op == MINT_OP_ALLGATHER ? op->world - 1
                      : allreduce                 ? 2 * op->world - 2
@@ -122,7 +130,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         if (rowwise && op->row_stride < op->count_bytes) return MINT_ERR_ARG;   // rows overlap
         if (op->total_bytes) {
             // rows cut from one buffer: the last ones may be short or empty
-            if (!rowwise || op->total_bytes % dt_size ||
+            if (!rowwise || alltoall || op->total_bytes % dt_size ||
                 op->total_bytes > (uint64_t)op->world * op->row_stride)
                 return MINT_ERR_ARG;
             a.total_bytes = op->total_bytes;
@@ -134,7 +142,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // which ranks need which buffers
     for (int p = 0; p < a.pipes && !plan->empty; ++p) {
         for (int h = 0; h <= a.hops; ++h) {
-            const int rank = a.cyc[(a.start[p] + h) % a.cyc_len];
+            const int rank = alltoall ? (h == 0 ? p / op->world : p % op->world)
+                                      : a.cyc[(a.start[p] + h) % a.cyc_len];
             const bool origin = h == 0, sink = h == a.hops;
             const bool load = allreduce ? h < op->world : origin || (reducing(op->op) && !sink);
             const bool save = allreduce ? h >= op->world - 1
@@ -146,6 +155,14 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
             if (!origin && (!op->staging[rank] || !aligned16(op->staging[rank])))
                 return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
         }
+    }
+    if (alltoall && !plan->empty) {
+        // every row is read while others are written: no output may overlap an input
+        const uint64_t extent = (uint64_t)(op->world - 1) * op->row_stride + op->count_bytes;
+        for (int i = 0; i < op->world; ++i)
+            for (int o = 0; o < op->world; ++o)
+                if (op->input[i] < op->output[o] + extent && op->output[o] < op->input[i] + extent)
+                    return MINT_ERR_ARG;
     }
     for (int r = 0; r < op->world; ++r) {
         a.input[r] = op->input[r];
@@ -159,7 +176,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // a slot is shared evenly by the pipelines, in whole 1 KiB blocks; what
     // does not divide is left unused
     if (op->slot_bytes % kBlockMsg) return MINT_ERR_GEOMETRY;
-    a.step_blocks = op->slot_bytes / kBlockMsg / (uint32_t)(a.pipes * a.phases);
+    a.step_blocks = op->slot_bytes / kBlockMsg / (uint32_t)a.shares;
     if (a.step_blocks == 0) return MINT_ERR_GEOMETRY;
     a.step_msg = a.step_blocks * kBlockMsg;
     if (op->waves_per_channel_group == 0 || a.step_blocks % op->waves_per_channel_group)
@@ -207,8 +224,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     if (op->placement == MINT_PLACE_LOCAL && (a.pipes * a.blocks_per_group) % kXcds)
         return MINT_ERR_GEOMETRY;
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
-    plan->staging_need = (size_t)a.credit_off +
-                         (size_t)a.pipes * (size_t)a.phases * (size_t)a.waves * kCreditStride;
+    plan->staging_need = (size_t)a.credit_off + (size_t)a.shares * (size_t)a.waves * kCreditStride;
     // The credit words lie behind the slots: a buffer that only holds the
     // slots (the reference's recvbuff is BUFF_SIZE bytes, 7_reducescatter.py:93)
     // would be written out of bounds.

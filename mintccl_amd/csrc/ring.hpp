@@ -16,7 +16,9 @@
 // 5_reduce.py:79-89, 7_reducescatter.py:57-67; here they are different
 // wavefronts, so nothing has to lag).  Allreduce is the same walk carried on:
 // 2 * world - 1 positions, the first `world` add, the rest copy, and every
-// position from the last adder on keeps the result.
+// position from the last adder on keeps the result.  Alltoall is world * world
+// pipelines of two positions: pipeline s * world + d carries row d of rank s
+// straight into row s of rank d (every pair of virtual ranks is linked).
 //
 // Each (pipeline, position) is served by W *wave-channels*; wave-channel w of
 // position h talks only to wave-channel w of positions h-1 and h+1.  Staging
@@ -40,7 +42,7 @@
 namespace mint {
 
 enum : int { OP_SENDRECV = 0, OP_BROADCAST = 1, OP_REDUCE = 2, OP_ALLGATHER = 3,
-             OP_REDUCESCATTER = 4, OP_ALLREDUCE = 5 };
+             OP_REDUCESCATTER = 4, OP_ALLREDUCE = 5, OP_ALLTOALL = 6 };
 enum : int { PROTO_LL128 = 0, PROTO_SIMPLE = 1 };
 enum : int { PLACE_SPREAD = 0, PLACE_LOCAL = 1 };
 
@@ -60,6 +62,7 @@ struct RingArgs {
     uint64_t row_bytes, row_stride;
     uint64_t total_bytes;                 // 0, or clip row p to total_bytes - p * row_stride
     int32_t phases;                       // staging shares per pipeline (2 for allreduce)
+    int32_t shares;                       // shares of a slot: pipes * phases; alltoall: one per source rank
     uint32_t nblocks;                     // blocks per row
     uint32_t steps;                       // steps per row
     uint32_t slot_bytes, nslots;
@@ -82,6 +85,16 @@ struct Role {
 
 __device__ __forceinline__ Role role_of(const RingArgs& a, int p, int h) {
     Role r;
+    if (a.op == OP_ALLTOALL) {
+        // pipeline p = source * world + destination: origin, then sink
+        const int src = p / a.world, dst = p % a.world;
+        r.rank = h == 0 ? src : dst;
+        r.next = dst;
+        r.load = r.send = h == 0;
+        r.recv = r.save = h != 0;
+        r.reduce = false;
+        return r;
+    }
     const int s = a.start[p];
     r.rank = a.cyc[(s + h) % a.cyc_len];
     r.next = a.cyc[(s + h + 1) % a.cyc_len];
@@ -221,7 +234,17 @@ __host__ __device__ __forceinline__ void row_extent(const RingArgs& a, int p, ui
 // is built, once while it is handed round): each phase has its own share of
 // the slots and its own credit words.
 __host__ __device__ __forceinline__ uint32_t share_of(const RingArgs& a, int p, int h) {
+    if (a.op == OP_ALLTOALL) return (uint32_t)(p / a.world);      // the source rank's share
     return (uint32_t)p * (uint32_t)a.phases + (h >= a.world && a.phases > 1 ? 1u : 0u);
+}
+// Rows of the caller's buffers a pipeline reads and writes: row p of every
+// rank, except alltoall, where pipeline source * world + destination reads row
+// `destination` of the source and writes row `source` of the destination.
+__host__ __device__ __forceinline__ uint32_t row_read(const RingArgs& a, int p) {
+    return a.op == OP_ALLTOALL ? (uint32_t)(p % a.world) : (uint32_t)p;
+}
+__host__ __device__ __forceinline__ uint32_t row_written(const RingArgs& a, int p) {
+    return a.op == OP_ALLTOALL ? (uint32_t)(p / a.world) : (uint32_t)p;
 }
 
 // How staging memory is accessed.  The sector tags make any choice safe: a
@@ -295,12 +318,13 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                                           const RoleT role, const LdsPort port = LdsPort{}) {
     constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
     const LaneMap m;
-    const uint64_t row_off = (uint64_t)p * a.row_stride;
     uint64_t row_bytes;
     uint32_t nblocks, nfull;
     row_extent(a, p, PROTO == PROTO_LL128 ? kBlockRawLL : kBlockRawSimple, row_bytes, nblocks, nfull);
-    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) + row_off;
-    uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) + row_off;
+    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[role.rank]) +
+                            (uint64_t)row_read(a, p) * a.row_stride;
+    uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[role.rank]) +
+                       (uint64_t)row_written(a, p) * a.row_stride;
     const uint32_t ring_bytes = a.nslots * a.slot_bytes;
     const Window own(reinterpret_cast<const void*>(a.staging[role.rank]), ring_bytes);
     const Window nxt(reinterpret_cast<const void*>(a.staging[role.next]), ring_bytes);

@@ -216,13 +216,30 @@ def allreduce() -> bool:
     return all([_report(r, bufs[r], want, r == 0) for r in range(world)])
 
 
+def alltoall() -> bool:
+    """The self-test the planned 9_alltoall would carry (README.md:24): the
+    second opinion is the transpose done with plain torch copies."""
+    from .alltoall import alltoall as op
+    comm = VirtualComm()
+    dev, world = comm.device, comm.world_size
+    n = common.test_count() // world
+    g = _gen(dev)
+    bufs = [torch.empty(world, n, device=dev).random_(generator=g) for _ in range(world)]
+    outs = [torch.zeros_like(b) for b in bufs]
+    _run_all(comm, lambda r: op(bufs[r], outs[r], comm))
+    if not common.test_mode():
+        return True
+    return all([_report(d, outs[d], torch.stack([bufs[s][d] for s in range(world)]), d == 0)
+                for d in range(world)])
+
+
 def main(name: str) -> int:
     from . import sendrecv_buffer, sendrecv_indirect
     tests = {"sendrecv_direct": sendrecv_direct,
              "sendrecv_indirect": lambda: sendrecv(sendrecv_indirect),
              "sendrecv_buffer": lambda: sendrecv(sendrecv_buffer),
              "broadcast": broadcast, "reduce": reduce, "allgather": allgather,
-             "reducescatter": reducescatter, "allreduce": allreduce}
+             "reducescatter": reducescatter, "allreduce": allreduce, "alltoall": alltoall}
     if name == "all":
         return 0 if all([fn() for fn in tests.values()]) else 1
     return 0 if tests[name]() else 1

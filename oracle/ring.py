@@ -176,6 +176,17 @@ def allreduce(xs: list, dtype: str, ring: list[int] | None = None) -> list:
     return [out.copy() for _ in xs]
 
 
+def alltoall(xs: list) -> list:
+    """xs[s] = rank s's ``(N, n)`` buffer (bytes).  Returns every rank's output:
+    row s of rank d is row d of rank s (MPI_Alltoall; the reference plans it
+    as ``9_alltoall.py``, ``README.md:24,50``, and holds no code for it).
+    Pinned by definition: a transpose of whole rows, bit-exact copies; applied
+    twice it gives the input back."""
+    n_ranks = len(xs)
+    rows = [_bytes(x).reshape(n_ranks, -1) for x in xs]
+    return [np.concatenate([rows[s][d] for s in range(n_ranks)]) for d in range(n_ranks)]
+
+
 def broadcast(xs: list, root: int) -> list:
     return [_bytes(xs[root]).copy() for _ in xs]
 

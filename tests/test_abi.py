@@ -117,13 +117,21 @@ def test_plan_geometry_without_a_gpu():
     d = make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=16, count_bytes=8 << 20)
     assert L.mint_ring_grid_blocks(d) == 8 * 15 * 4
     assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 2 * 16 * 256
+    # alltoall: 64 pipelines x 2 positions; a slot has one share per source rank
+    d = make_op(op=_lib.OP_ALLTOALL, dtype=_lib.BYTES, waves_per_channel_group=16)
+    for r in range(8):
+        d.output[r] = 0x40000000 + r * 0x1000000
+    assert L.mint_ring_grid_blocks(d) == 64 * 2 * 4
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256
+    d.output[5] = d.input[2] + (3 << 20)                    # an output inside an input
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=64)) \
         == _lib.ERR_GEOMETRY          # 512 KiB slot / 16 shares = 32 blocks per step
 
 
 @pytest.mark.parametrize("kw,err", [
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
-    (dict(op=6), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=7), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
     (dict(dtype=_lib.BYTES), _lib.ERR_ARG),          # a reduction needs a real dtype
     (dict(flag_epoch=0), _lib.ERR_ARG), (dict(flag_epoch=4096), _lib.ERR_ARG),
     (dict(status=0), _lib.ERR_ARG), (dict(cache_policy=3), _lib.ERR_ARG),

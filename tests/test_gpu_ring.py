@@ -142,6 +142,46 @@ def test_reduce_and_allreduce_with_own_rows_through_lds(dev, world):
     assert same(bufs, ring.broadcast(raw, 0))
 
 
+@pytest.mark.parametrize("proto", [0, 1])
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("n", [1, 479, 480, 481, 100003])
+def test_alltoall(dev, proto, world, n):
+    """Row d of rank s arrives as row s of rank d, bit for bit, and the inputs
+    are left alone (oracle: the transpose of rows)."""
+    from mintccl_amd.alltoall import alltoall
+    host = [uniform(world * n, -1.0, 1.0, 70 + r).reshape(world, n) for r in range(world)]
+    want = ring.alltoall([as_bytes(h) for h in host])
+    for kw in (dict(), dict(buff_size_=world * 8 * 3072, nslots=3, waves_per_rank=2 * 8 * world)):
+        bufs = [h.to(dev) for h in host]
+        outs = [torch.full_like(b, 7.0) for b in bufs]
+        comm = make_comm(world, protocol=proto, **kw)
+        comm.run(lambda r: alltoall(bufs[r], outs[r], comm))
+        comm.check()
+        assert same(outs, want), kw
+        assert same(bufs, [as_bytes(h) for h in host])
+
+
+def test_alltoall_64mib_and_argument_checks(dev):
+    from mintccl_amd.alltoall import alltoall
+    world, n = 8, 4194304                                   # 8 ranks x 64 MiB fp16
+    bufs = []
+    for r in range(world):
+        g = torch.Generator(device=dev).manual_seed(90 + r)
+        bufs.append(torch.randn(world, n, generator=g, device=dev, dtype=torch.float16))
+    outs = [torch.zeros_like(b) for b in bufs]
+    comm = make_comm(world)
+    comm.run(lambda r: alltoall(bufs[r], outs[r], comm))
+    comm.check()
+    for d in range(world):
+        for s in range(world):
+            assert torch.equal(outs[d][s].view(torch.int16), bufs[s][d].view(torch.int16)), (d, s)
+    with comm.rank(0):
+        with pytest.raises(ValueError):
+            alltoall(bufs[0], outs[0][:, : n // 2].contiguous(), comm)        # sizes differ
+    with pytest.raises(ValueError):
+        comm.run(lambda r: alltoall(bufs[r], bufs[(r + 1) % world], comm))    # out is somebody's buff
+
+
 def test_reducescatter_special_values(dev):
     # overflow to inf, inf - inf, subnormals, signed zeros ride the ring unharmed
     world, n = 4, 960

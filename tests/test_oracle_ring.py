@@ -237,3 +237,17 @@ def test_torch_cpu_walk_equals_the_numpy_walk(dt, world, n):
         assert ring.reducescatter(raw, dt, ring=rg)[0].tobytes() == want[0].tobytes()
         for r in range(world):
             assert np.array_equal(got[r].view(torch.uint8).numpy().reshape(-1), want[r]), r
+
+
+def test_alltoall_is_the_transpose_of_rows():
+    # hand-written: 3 ranks, rows of two bytes; rank s row d = (10 s + d) twice
+    xs = [np.array([[10 * s + d] * 2 for d in range(3)], dtype=np.uint8).reshape(-1) for s in range(3)]
+    out = ring.alltoall(xs)
+    assert out[0].tolist() == [0, 0, 10, 10, 20, 20]
+    assert out[1].tolist() == [1, 1, 11, 11, 21, 21]
+    assert out[2].tolist() == [2, 2, 12, 12, 22, 22]
+    rng = np.random.default_rng(3)
+    xs = [rng.integers(0, 256, 5 * 37, dtype=np.uint8) for _ in range(5)]
+    twice = ring.alltoall(ring.alltoall(xs))
+    assert all(np.array_equal(a, b) for a, b in zip(twice, xs))          # an involution
+    assert sum(int(x.sum()) for x in xs) == sum(int(x.sum()) for x in ring.alltoall(xs))

@@ -120,3 +120,31 @@ def test_rows_clipped_to_one_buffer():
     for p, left in enumerate([row] * 5 + [2000, 0, 0]):
         blocks = np.concatenate([schedule(d, p, 1, w)[1] for w in range(16)])
         assert sorted(blocks.tolist()) == list(range(-(-left // 960)))
+
+
+def test_alltoall_shares_are_per_source_rank():
+    """Alltoall: pipeline s * world + d; rank d's slots have one share per
+    source rank, so what the origin of (s, d) sends lands in share s of d's
+    slot - for every s a different part - and every block goes once."""
+    d = make_op(op=_lib.OP_ALLTOALL, dtype=_lib.BYTES, count_bytes=(1 << 20) + 16,
+                waves_per_channel_group=16)
+    for r in range(8):
+        d.output[r] = 0x40000000 + r * 0x1000000
+    d.row_stride = d.count_bytes
+    assert _lib.lib().mint_ring_grid_blocks(d) == 64 * 2 * 4
+    nblocks = -(-d.count_bytes // 960)
+    share = d.slot_bytes // 1024 // 8 * 1024
+    for s, dst in ((0, 0), (3, 5), (7, 2)):
+        p = s * 8 + dst
+        seen = np.zeros(nblocks, dtype=np.int64)
+        for w in range(16):
+            step, block, _, send = schedule(d, p, 0, w)
+            step1, block1, recv, _ = schedule(d, p, 1, w)
+            np.add.at(seen, block, 1)
+            assert np.array_equal(block, block1) and np.array_equal(send, recv)
+            assert np.all((send % d.slot_bytes) // share == s)
+            assert np.array_equal(send // d.slot_bytes, step % d.nslots)
+        assert np.all(seen == 1)
+    n = ctypes.c_uint32(0)
+    assert _lib.lib().mint_ring_schedule(d, 64, 0, 0, 0, None, None, None, None,
+                                         ctypes.byref(n)) == _lib.ERR_ARG
