@@ -60,6 +60,11 @@ THREADS = int(os.getenv("MINTCCL_BENCH_THREADS", 256))
 PLACEMENT = int(os.getenv("MINTCCL_BENCH_PLACEMENT", 1))      # 0 spread, 1 local
 CACHE_POLICY = int(os.getenv("MINTCCL_BENCH_CACHE", 2))       # 0 agent, 1 system, 2 XCD-local
 ROW_FETCH = int(os.getenv("MINTCCL_BENCH_FETCH", 0))          # 0 in registers, 1 through LDS
+# Diagnostic: run on a stream restricted to some of the CUs (hex pattern of 32
+# bits, repeated over the device's CUs; 00FF00FF leaves half of the CUs of
+# every XCD) to tell a per-CU limit from a device-wide one.  A grid that is no
+# longer co-resident still finishes: a channel's positions are dispatched together.
+CU_MASK = os.getenv("MINTCCL_BENCH_CU_MASK", "")
 
 
 def geometry_key() -> str:
@@ -157,6 +162,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--also-64mib", action="store_true",
+                    help="also time the same collective at 64 MiB per rank (the baseline's "
+                         "configuration 4 reading of the headline); off by default so that every "
+                         "launch of the ring kernel in a profile of this command is a headline launch")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.getenv("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the 8 ring ranks are disjoint HBM regions "
@@ -170,6 +179,15 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if CU_MASK:
+        import ctypes
+        hip = ctypes.CDLL("libamdhip64.so")
+        words = (ctypes.c_uint32 * 8)(*([int(CU_MASK, 16)] * 8))
+        handle = ctypes.c_void_p()
+        if hip.hipExtStreamCreateWithCUMask(ctypes.byref(handle), 8, words) != 0:
+            print("bench.py: hipExtStreamCreateWithCUMask failed", file=sys.stderr)
+            return 1
+        torch.cuda.set_stream(torch.cuda.ExternalStream(handle.value))
 
     # yardsticks: the library's own copy and read-only kernels on 1 GiB
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256)
@@ -229,25 +247,27 @@ def main() -> int:
     comm.check()
     kernel_ms = sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / args.steps
 
-    # the other reading of the baseline's headline (its config 4: 32 Mi
-    # elements = 64 MiB per rank), same launch geometry, labelled as such
-    small = [b[:, : n // 4] .contiguous() for b in bufs]
+    small_ms = None
+    if args.also_64mib:
+        # the other reading of the baseline's headline (its config 4: 32 Mi
+        # elements = 64 MiB per rank), same launch geometry, labelled as such
+        small = [b[:, : n // 4] .contiguous() for b in bufs]
 
-    def small_step():
-        comm.run(lambda r: reducescatter(small[r], comm))
+        def small_step():
+            comm.run(lambda r: reducescatter(small[r], comm))
 
-    for _ in range(args.warmup):
-        small_step()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(args.steps):
-        small_step()
-    e1.record()
-    torch.cuda.synchronize()
-    comm.check()
-    small_ms = e0.elapsed_time(e1) / args.steps
-    del small
+        for _ in range(args.warmup):
+            small_step()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            small_step()
+        e1.record()
+        torch.cuda.synchronize()
+        comm.check()
+        small_ms = e0.elapsed_time(e1) / args.steps
+        del small
 
     # the loads and stores of the same launch with nothing waiting for anything
     wave_channels = WAVES_PER_RANK * (WORLD + 1)          # one per (chunk, position, channel)
@@ -282,7 +302,7 @@ def main() -> int:
                    "nslots": NSLOTS, "waves_per_rank": WAVES_PER_RANK, "threads": THREADS,
                    "placement": ["spread", "local"][PLACEMENT],
                    "staging_cache_policy": ["agent", "system", "xcd-local"][CACHE_POLICY],
-                   "own_rows": ["registers", "lds"][ROW_FETCH],
+                   "own_rows": ["registers", "lds"][ROW_FETCH], "cu_mask": CU_MASK or None,
                    "grid_blocks": comm.last_grid, "hbm_bytes_per_step": hbm_bytes,
                    "payload_bytes_per_step": payload},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
@@ -307,11 +327,12 @@ def main() -> int:
                              "no waiting (mint_step_mix)"},
         "algbw_gbps": round(algbw, 1), "busbw_gbps": round(algbw * (WORLD - 1) / WORLD, 1),
         "flag_bytes_frac_of_staging": round(8 / 128, 4),
-        "at_64mib_per_rank": {"workload": "same collective, 64 MiB fp16 per rank (32 Mi elements)",
-                              "ms_per_step": round(small_ms, 4),
-                              "hbm_gbps": round((WORLD + 1) * (PER_RANK_BYTES // 4)
-                                                / (small_ms / 1e3) / 1e9, 1)},
     }
+    if small_ms is not None:
+        out["at_64mib_per_rank"] = {
+            "workload": "same collective, 64 MiB fp16 per rank (32 Mi elements)",
+            "ms_per_step": round(small_ms, 4),
+            "hbm_gbps": round((WORLD + 1) * (PER_RANK_BYTES // 4) / (small_ms / 1e3) / 1e9, 1)}
     if not args.no_cpu_baseline:
         out.update(cpu_baselines())
     print(json.dumps(out))

@@ -10,10 +10,19 @@ adder folded in ring order).
   config 3  ring broadcast 64 MiB, 8 ranks, 8 x 512 KiB slots
   config 4  ring reduce and reducescatter, 32 Mi elements per rank, f16 / bf16 / f32
   config 5  ring allgather sweep, shard 512 B .. 128 MiB, LL128 vs Simple
-  next      ring allreduce (the reference's planned 8_allreduce), 64 and 256 MiB fp16
+  next      ring allreduce (the reference's planned 8_allreduce), 64 and 256 MiB fp16;
+            alltoall (its planned 9_alltoall), 64 and 256 MiB fp16 per rank
 
-Algorithmic bytes: copy 2S; sendrecv over h hops
-(2 + 2h) S; broadcast / allgather (3N - 2) S; reduce / reducescatter (3N + 1) S.
+    --staging reference|tuned   only the geometry the configuration names, or
+                                only the library's tuned default (a profile of one
+                                such run has one launch shape per kernel name)
+
+Algorithmic bytes (`alg_gbps`: what the ring moves, staging included): copy 2S;
+sendrecv over h hops (2 + 2h) S; broadcast / allgather (3N - 2) S; reduce /
+reducescatter (3N + 1) S; alltoall 4 N S.  `hbm_gbps` counts only what has to
+cross HBM - inputs read once, results written once: sendrecv 2S, broadcast N S,
+allgather N S (S = N shards), reduce / reducescatter (N + 1) S, allreduce
+2 N S, alltoall 2 N S.
 """
 from __future__ import annotations
 
@@ -56,7 +65,24 @@ def time_ms(fn, reps: int) -> float:
     return best
 
 
+STAGING = ("reference", "tuned")      # set from --staging
+
+
+def geometries(reference_label: str, slots):
+    """(label, slots) pairs to run: the geometry the configuration names and /
+    or the library's tuned default."""
+    out = []
+    if "reference" in STAGING:
+        out.append((reference_label, slots))
+    if "tuned" in STAGING:
+        out.append(("tuned", None))
+    return out
+
+
 def emit(**kw) -> None:
+    if "hbm_bytes" in kw:
+        t = kw["ms"] if "ms" in kw else kw["us"] / 1e3
+        kw["hbm_gbps"] = round(kw.pop("hbm_bytes") / t / 1e6, 1)
     print(json.dumps(kw), flush=True)
 
 
@@ -75,7 +101,7 @@ def config2(reps: int) -> None:
     dst = torch.zeros_like(src)
     S = n * 2
     for name, proto in (("ll128", 0), ("simple", 1)):
-        for label, slots in (("8x512KiB", (8, 512 * 1024)), ("tuned", None)):
+        for label, slots in geometries("8x512KiB", (8, 512 * 1024)):
             comm = comm_for(2, proto, slots, waves_per_rank=512 if slots else None)
 
             def step():
@@ -91,8 +117,8 @@ def config2(reps: int) -> None:
             ok = torch.equal(dst.view(torch.int16), src.view(torch.int16))
             ms = time_ms(step, reps)
             emit(config=2, op="sendrecv", protocol=name, staging=label, bytes=S, ms=round(ms, 4),
-                 alg_gbps=round(4 * S / ms / 1e6, 1), algbw_gbps=round(S / ms / 1e6, 1), ok=ok,
-                 grid=comm.last_grid)
+                 alg_gbps=round(4 * S / ms / 1e6, 1), hbm_bytes=2 * S,
+                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
     comm = VirtualComm(world_size=2, device=DEV)
 
     def direct():
@@ -107,7 +133,7 @@ def config2(reps: int) -> None:
     ok = torch.equal(dst.view(torch.int16), src.view(torch.int16))
     ms = time_ms(direct, reps)
     emit(config=2, op="sendrecv_direct", protocol="simple copy", bytes=S, ms=round(ms, 4),
-         alg_gbps=round(2 * S / ms / 1e6, 1), algbw_gbps=round(S / ms / 1e6, 1), ok=ok)
+         alg_gbps=round(2 * S / ms / 1e6, 1), hbm_bytes=2 * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok)
 
 
 def config3(reps: int) -> None:
@@ -117,7 +143,7 @@ def config3(reps: int) -> None:
     bufs = [root.clone() if r == 0 else torch.zeros_like(root) for r in range(world)]
     S = n * 2
     for name, proto in (("ll128", 0), ("simple", 1)):
-        for label, slots in (("8x512KiB", (8, 512 * 1024)), ("tuned", None)):
+        for label, slots in geometries("8x512KiB", (8, 512 * 1024)):
             comm = comm_for(world, proto, slots, waves_per_rank=512 if slots else None)
             for b in bufs[1:]:
                 b.zero_()
@@ -131,7 +157,7 @@ def config3(reps: int) -> None:
             ms = time_ms(step, reps)
             emit(config=3, op="broadcast", protocol=name, staging=label, world=world, bytes=S,
                  ms=round(ms, 4), alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1),
-                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+                 hbm_bytes=world * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
 
 
 def fold_device(rows: list, order: list[int]) -> torch.Tensor:
@@ -151,7 +177,7 @@ def config4(reps: int) -> None:
             orig.append(torch.randn(world, n, generator=g, device=DEV, dtype=torch.float32)
                         .to(TDT[dt]))
         S = n_total * orig[0].element_size()
-        for label, slots in (("8x1MiB", (8, 1 << 20)), ("tuned", None)):
+        for label, slots in geometries("8x1MiB", (8, 1 << 20)):
             comm = comm_for(world, 0, slots, waves_per_rank=512 if slots else None)
             bufs = [o.clone() for o in orig]
 
@@ -167,7 +193,7 @@ def config4(reps: int) -> None:
             ms = time_ms(rs, reps)
             emit(config=4, op="reducescatter", dtype=dt, staging=label, world=world, bytes=S,
                  ms=round(ms, 4), alg_gbps=round((3 * world + 1) * S / ms / 1e6, 1),
-                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+                 hbm_bytes=(world + 1) * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
             flat = [o.reshape(-1).clone() for o in orig]
 
             def rd():
@@ -181,14 +207,14 @@ def config4(reps: int) -> None:
             ms = time_ms(rd, reps)
             emit(config=4, op="reduce", dtype=dt, staging=label, world=world, bytes=S,
                  ms=round(ms, 4), alg_gbps=round((3 * world + 1) * S / ms / 1e6, 1),
-                 algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
+                 hbm_bytes=(world + 1) * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
 
 
 def config5(reps: int, max_log2: int) -> None:
     world = 8
     for name, proto in (("ll128", 0), ("simple", 1)):
-        comms = {"8x512KiB": comm_for(world, proto, (8, 512 * 1024), waves_per_rank=512),
-                 "tuned": comm_for(world, proto, None)}
+        comms = {label: comm_for(world, proto, slots, waves_per_rank=512 if slots else None)
+                 for label, slots in geometries("8x512KiB", (8, 512 * 1024))}
         for log2 in range(9, max_log2 + 1):
             shard = 1 << log2
             n = shard // 2
@@ -216,7 +242,7 @@ def config5(reps: int, max_log2: int) -> None:
                 S = world * shard
                 emit(config=5, op="allgather", protocol=name, staging=label, world=world,
                      shard_bytes=shard, us=round(ms * 1e3, 2),
-                     alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1),
+                     alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1), hbm_bytes=world * S,
                      busbw_gbps=round(shard * (world - 1) / ms / 1e6, 1), ok=ok)
             del bufs
 
@@ -257,17 +283,56 @@ def allreduce_bench(reps: int) -> None:
             emit(config="next", op="allreduce", protocol=name,
                  mode="one pass" if fused else "reducescatter + allgather", staging="tuned",
                  world=world, bytes=S, ms=round(ms, 4), alg_gbps=round((6 * world - 4) * S / ms / 1e6, 1),
-                 algbw_gbps=round(S / ms / 1e6, 1),
+                 hbm_bytes=2 * world * S, algbw_gbps=round(S / ms / 1e6, 1),
                  busbw_gbps=round(2 * (world - 1) / world * S / ms / 1e6, 1), ok=ok,
                  grid=comm.last_grid)
         del orig
 
 
+def alltoall_bench(reps: int) -> None:
+    """The reference's planned 9_alltoall: 8 ranks, 64 and 256 MiB fp16 per
+    rank, every row straight into its destination's staging and out again
+    (per rank S read, S staged, S taken out of staging, S written: 4 N S)."""
+    from mintccl_amd.alltoall import alltoall
+    world = 8
+    for n_total in (33554432, 134217728):
+        n = n_total // world
+        bufs = []
+        for r in range(world):
+            g = torch.Generator(device=DEV).manual_seed(90 + r)
+            bufs.append(torch.randn(world, n, generator=g, device=DEV, dtype=torch.float32)
+                        .to(torch.float16))
+        outs = [torch.zeros_like(b) for b in bufs]
+        S = n_total * 2
+        for name, proto in (("ll128", 0), ("simple", 1)):
+            comm = comm_for(world, proto, None)
+
+            def step():
+                comm.run(lambda r: alltoall(bufs[r], outs[r], comm))
+
+            for o in outs:
+                o.zero_()
+            step()
+            comm.check()
+            ok = all(torch.equal(outs[d][s].view(torch.int16), bufs[s][d].view(torch.int16))
+                     for d in range(world) for s in range(world))
+            ms = time_ms(step, reps)
+            emit(config="next", op="alltoall", protocol=name, staging="tuned", world=world, bytes=S,
+                 ms=round(ms, 4), alg_gbps=round(4 * world * S / ms / 1e6, 1),
+                 hbm_bytes=2 * world * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok,
+                 grid=comm.last_grid)
+        del bufs, outs
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--staging", choices=("both", "reference", "tuned"), default="both")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
-    ap.add_argument("--only", type=int, default=0, help="run one config (2..5; 8 = allreduce)")
+    ap.add_argument("--only", type=int, default=0,
+                    help="run one config (2..5; 8 = allreduce; 9 = alltoall)")
     args = ap.parse_args()
+    global STAGING
+    STAGING = ("reference", "tuned") if args.staging == "both" else (args.staging,)
     reps = 3 if args.quick else 8
     torch.cuda.set_device(DEV)
     if args.only in (0, 2):
@@ -280,6 +345,8 @@ def main() -> int:
         config5(reps, 24 if args.quick else 27)
     if args.only in (0, 8):
         allreduce_bench(reps)
+    if args.only in (0, 9):
+        alltoall_bench(reps)
     return 0
 
 
