@@ -110,13 +110,16 @@ class Timer:
 
 
 # Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
-# step.  Collectives with one pipeline per rank (allgather, reducescatter,
-# allreduce): 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in all
+# step.  The copying collectives with one pipeline per rank (allgather,
+# alltoall): 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in all
 # (from about 6100 on the grid no longer runs as one wave of blocks and the
-# time jumps by a third).  Collectives with a single pipeline (sendrecv,
-# broadcast, reduce): 3 slots of 512 KiB, 4608 wavefronts; a slot may grow to
-# TUNED_SLOT_BUDGET bytes when there are few hops.  Staging is allocated for
-# TUNED_NSLOTS slots of TUNED_SLOT_BUDGET either way.
+# time jumps by a third).  Everything else - the collectives with a single
+# pipeline (sendrecv, broadcast, reduce) and the reducing ones (reducescatter,
+# allreduce): 3 slots of 512 KiB, 4608 wavefronts; a slot may grow to
+# TUNED_SLOT_BUDGET bytes when there are few hops.  The reducing collectives
+# run thread blocks of 2 wave-channels (TUNED_THREADS_REDUCING) unless the
+# caller names a block size.  Staging is allocated for TUNED_NSLOTS slots of
+# TUNED_SLOT_BUDGET either way.
 TUNED_TOTAL_WAVES = 4608
 TUNED_SLOT_BLOCKS = 512
 TUNED_NSLOTS = 3
@@ -124,6 +127,7 @@ TUNED_TOTAL_WAVES_MULTI = 5760
 TUNED_SLOT_BLOCKS_MULTI = 640
 TUNED_NSLOTS_MULTI = 2
 TUNED_SLOT_BUDGET = 2304 * 1024
+TUNED_THREADS_REDUCING = 128
 
 
 class RingTimeout(RuntimeError):
@@ -146,7 +150,8 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         # per source rank
         total = TUNED_TOTAL_WAVES_MULTI
         wpb = max(1, threads_per_block // 64)
-        waves = max(wpb, total // (2 * world * world) // wpb * wpb)
+        granule = wpb * (8 // math.gcd(world * world, 8))      # whole channels for every XCD
+        waves = max(granule, total // (2 * world * world) // granule * granule)
         return world * waves * 1024, min(max_nslots, TUNED_NSLOTS_MULTI), waves
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
     real_pipes = pipes
@@ -159,7 +164,7 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         npos = (npos + 1) // 2    # `pipes` already counts both phases
     # slots sized per 8 receiving ranks keep the staging of an XCD's channels
     # (slots x receivers / 8) well inside its 4 MiB of L2
-    multi = real_pipes > 1
+    multi = op == _lib.OP_ALLGATHER
     per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
     total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
     wpb = max(1, threads_per_block // 64)
@@ -247,6 +252,7 @@ class VirtualComm:
             waves_per_rank = (max(1, num_blocks() * num_warps() // 2) if reference_geometry
                               else 512)
         self.waves_per_rank = waves_per_rank
+        self.threads_explicit = threads_per_block is not None or bool(os.getenv("MINTCCL_THREADS"))
         self.threads_per_block = (threads_per_block if threads_per_block is not None
                                   else _env_int("MINTCCL_THREADS", 256))
         if cache_policy is None:
@@ -357,12 +363,15 @@ class VirtualComm:
                                           _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL) else 1
         if op == _lib.OP_ALLREDUCE:
             pipes *= 2            # a slot is shared by (pipeline, phase): two phases
+        threads = self.threads_per_block
+        reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
         if self.auto_geometry:
             lds = (self.row_fetch == _lib.FETCH_LDS and d.protocol == _lib.PROTO_LL128
-                   and op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
-                   and self.threads_per_block // 64 in (4, 7))
+                   and reducing and threads // 64 in (4, 7))
+            if reducing and not lds and not self.threads_explicit:
+                threads = TUNED_THREADS_REDUCING
             d.slot_bytes, d.nslots, d.waves_per_channel_group = tuned_geometry(
-                op, self.world_size, route_len, self.threads_per_block, self.nslots, lds)
+                op, self.world_size, route_len, threads, self.nslots, lds)
         else:
             d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
             step_blocks = self.slot_bytes // 1024 // pipes
@@ -374,13 +383,13 @@ class VirtualComm:
             groups = 2 * pipes if op == _lib.OP_ALLTOALL else pipes
             d.waves_per_channel_group = _largest_divisor_at_most(
                 step_blocks, max(1, self.waves_per_rank // groups))
-        d.threads_per_block = self.threads_per_block
+        d.threads_per_block = threads
         d.placement, d.cache_policy = self.placement, self.cache_policy
         d.row_fetch = self.row_fetch
         if self.placement == _lib.PLACE_LOCAL:
             # whole channels are dealt to the 8 XCDs; when the channel count
             # does not divide, this launch runs spread with agent-scope staging
-            wpb = max(1, min(self.threads_per_block // 64, d.waves_per_channel_group))
+            wpb = max(1, min(threads // 64, d.waves_per_channel_group))
             real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
             if op == _lib.OP_ALLTOALL:
                 real_pipes = self.world_size * self.world_size

@@ -415,19 +415,20 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         return true;
     };
 
-    // Own rows of the group being handled (v) and of the one fetched ahead
-    // (vnext).  The copy at the end of a group makes the group wait for the
-    // fetch it has issued after its polls, so a wave-channel never runs more
-    // than one fetch ahead of the ring.  That is on purpose.  Measured against
-    // two buffers that swap roles (loop unrolled by two, no wait at the end):
-    // the wave-channels then run ahead, arrive early at their polls and
-    // credit words, re-poll three times as often (0.19 - 0.78 re-polls per
-    // group instead of 0.01 - 0.26) and the launch takes 0.82 ms instead of
-    // 0.76: the L2 request rate, not a wavefront's latency, bounds the kernel,
-    // and every failed poll is eight more requests.
-    u32x4 v[U], vnext[U];
+    // Own rows of the group being handled and of the one fetched ahead: two
+    // register buffers that swap roles from one whole group to the next (the
+    // loop over whole groups is unrolled by two).  Copying the fetched-ahead
+    // rows into place at the end of a group instead makes every group wait
+    // for the fetch it has just issued (a wait for all outstanding loads at
+    // the loop's end): a wave-channel's own work per step was 0.80 us that
+    // way and is 0.31 us this way.  What that buys depends on the launch
+    // geometry - with two slots the wave-channels only arrive earlier at
+    // their polls and credit words and re-poll more (0.82 ms against 0.76 for
+    // the 8 x 256 MiB reduce-scatter); with three smaller slots they have the
+    // slack to use it (0.71 ms), which is the tuned geometry.
+    u32x4 rows[2][U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) v[u] = vnext[u] = u32x4{0u, 0u, 0u, 0u};
+    for (int u = 0; u < U; ++u) rows[0][u] = rows[1][u] = u32x4{0u, 0u, 0u, 0u};
     Group q = Group::first_of(geom);
     uint32_t n = 0;
     // Loop-carried, and looked at in every iteration whether or not a credit
@@ -444,8 +445,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // flight: it has a whole group's time to come back from HBM.  The other
     // groups (the ragged end of a row, a step that is only partly filled) take
     // the guarded body and load their own rows on the spot.
-    auto run_group = [&](auto whole_tag) -> bool {
+    auto run_group = [&](auto whole_tag, auto parity_tag) -> bool {
         constexpr bool WHOLE = decltype(whole_tag)::value;
+        constexpr int P = decltype(parity_tag)::value;
+        u32x4 (&v)[U] = rows[P];
+        u32x4 (&vnext)[U] = rows[P ^ 1];
         const Group qn = q.next(geom);
         const uint32_t s = q.step;
         const uint32_t tag = (epoch << 20) | (s + 1u);
@@ -571,10 +575,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     else st64_agent(nxt_head, flag_hi | (uint64_t)(s + 1));
                 }
             }
-        }
-        if (WHOLE && !LDSF) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = vnext[u];
         }
         q = qn;
         ++n;
@@ -737,11 +737,16 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     }
 
     // block numbers grow from group to group, so the whole groups come first
-    if (!LDSF && role.load && n < ngroups && q.g[U - 1] < nfull) fetch_ahead(q, v);
-    while (n < ngroups && q.g[U - 1] < nfull)
-        if (!run_group(std::true_type{})) return;
+    using Even = std::integral_constant<int, 0>;
+    using Odd = std::integral_constant<int, 1>;
+    if (!LDSF && role.load && n < ngroups && q.g[U - 1] < nfull) fetch_ahead(q, rows[0]);
+    while (n < ngroups && q.g[U - 1] < nfull) {
+        if (!run_group(std::true_type{}, Even{})) return;
+        if (!(n < ngroups && q.g[U - 1] < nfull)) break;
+        if (!run_group(std::true_type{}, Odd{})) return;
+    }
     while (n < ngroups)
-        if (!run_group(std::false_type{})) return;
+        if (!run_group(std::false_type{}, Even{})) return;
 
     if (timing && lane_id() == 0) {
         unsigned long long* st = reinterpret_cast<unsigned long long*>(a.stats) + 8 * h;

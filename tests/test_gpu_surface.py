@@ -187,9 +187,9 @@ def test_reference_style_self_tests_pass(monkeypatch, capsys, world, count):
     assert selftest.main("all") == 0
     out = capsys.readouterr().out
     assert "equal: False" not in out
-    # 3 point-to-point tests, broadcast and allgather and allreduce on every rank,
-    # reduce at the root, reducescatter on every rank
-    assert out.count("equal: True") == 3 + 3 * world + 1 + world
+    # 3 point-to-point tests, broadcast, allgather, allreduce and alltoall on every
+    # rank, reduce at the root, reducescatter on every rank
+    assert out.count("equal: True") == 3 + 4 * world + 1 + world
 
 
 @pytest.mark.gpu

@@ -31,19 +31,23 @@ def test_largest_divisor(n, cap, want):
 
 @pytest.mark.parametrize("world", [2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("op", [_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_REDUCE, _lib.OP_ALLGATHER,
-                                _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE])
+                                _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL])
 def test_tuned_geometry_is_always_launchable(op, world):
     """Whatever the collective and the world size, the tuned geometry passes the
     library's own plan check, deals whole channels to the 8 XCDs, fits its
     staging budget and stays inside the wavefront budget."""
     from tests.test_abi import make_op
-    slot, nslots, waves = common.tuned_geometry(op, world, 2, 256, common.TUNED_NSLOTS)
+    reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
+    threads = common.TUNED_THREADS_REDUCING if reducing else 256
+    slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS)
     assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
-    multi = op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
+    multi = op in (_lib.OP_ALLGATHER, _lib.OP_ALLTOALL)
     d = make_op(op=op, world=world, slot_bytes=slot, nslots=nslots, waves_per_channel_group=waves,
-                placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2,
-                dtype=_lib.F16 if op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
-                else _lib.BYTES)
+                placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2, threads_per_block=threads,
+                dtype=_lib.F16 if reducing else _lib.BYTES)
+    if op == _lib.OP_ALLTOALL:
+        for r in range(8):
+            d.output[r] = 0x40000000 + r * 0x1000000
     for i in range(9):
         d.ring[i] = i % world if i < world else 0
     d.ring[world] = 0
@@ -54,9 +58,12 @@ def test_tuned_geometry_is_always_launchable(op, world):
     blocks = _lib.lib().mint_ring_grid_blocks(d)
     assert blocks > 0, blocks
     assert blocks % 8 == 0
-    assert blocks * 4 <= (common.TUNED_TOTAL_WAVES_MULTI if multi else common.TUNED_TOTAL_WAVES)
+    assert blocks * (threads // 64) <= (common.TUNED_TOTAL_WAVES_MULTI if multi
+                                        else common.TUNED_TOTAL_WAVES)
 
 
 def test_headline_geometry():
-    assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
+    assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 128, 3) == (512 * 1024, 3, 64)
+    assert common.tuned_geometry(_lib.OP_ALLREDUCE, 8, 0, 128, 3) == (512 * 1024, 3, 32)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
