@@ -197,6 +197,8 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
  *   2  a 16-byte-per-lane agent-scope load of 1 KiB from one of the wave's two
  *      private slots in `staging` (needs waves * 2048 bytes, 16-byte aligned),
  *   4  a 16-byte-per-lane store of the f16 sum of the two into the other slot,
+ *   8  (with 1) the own block is loaded straight into LDS (buffer_load ... lds)
+ *      and read from there, instead of into registers,
  * with no flags and nobody waiting for anybody.  The launch takes what the
  * device needs for that mix of accesses however well a ring schedules them:
  * the yardstick beside mint_copy_simple and mint_read_xor.  `sink` (device

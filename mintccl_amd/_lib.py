@@ -12,7 +12,9 @@ import subprocess
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_PKG)
-SO_PATH = os.path.join(_PKG, "libmintccl.so")
+# MINTCCL_LIBRARY points at a diagnostic build (see build(defines=...)); it has
+# to exist like the in-tree one.
+SO_PATH = os.getenv("MINTCCL_LIBRARY") or os.path.join(_PKG, "libmintccl.so")
 _CSRC = os.path.join(_PKG, "csrc")
 SRC = os.path.join(_CSRC, "mintccl.hip")
 FAMILY_SRC = os.path.join(_CSRC, "ring_family.hip")     # compiled once per element type
@@ -102,16 +104,22 @@ SYMBOLS = {
 _lib = None
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | None = None) -> str:
     """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree).
 
     The ring kernels are one translation unit per element type; the five
-    compilations run side by side and are linked at the end."""
-    os.makedirs(BUILD_DIR, exist_ok=True)
-    units = [(SRC, [], os.path.join(BUILD_DIR, "mintccl.o"))]
+    compilations run side by side and are linked at the end.  ``defines``
+    (``-DMINT_RING_STATS``: wait accounting per ring position,
+    ``-DMINT_EARLY_POLL_ALL``: the adding kernels poll a step ahead like the
+    copying ones) and ``so_path`` make a diagnostic build beside the product's;
+    ``MINTCCL_LIBRARY`` loads it."""
+    out = so_path or os.path.join(_PKG, "libmintccl.so")
+    build_dir = BUILD_DIR if so_path is None else out + ".objs"
+    os.makedirs(build_dir, exist_ok=True)
+    units = [(SRC, list(defines), os.path.join(build_dir, "mintccl.o"))]
     for dt in range(4):
-        units.append((FAMILY_SRC, [f"-DMINT_FAMILY_DT={dt}"],
-                      os.path.join(BUILD_DIR, f"ring_family_{dt}.o")))
+        units.append((FAMILY_SRC, [f"-DMINT_FAMILY_DT={dt}", *defines],
+                      os.path.join(build_dir, f"ring_family_{dt}.o")))
     procs = []
     for src, defs, obj in units:
         cmd = ["hipcc", *HIPCC_FLAGS, *defs, "-c", "-o", obj, src]
@@ -126,14 +134,14 @@ def build(verbose: bool = False) -> str:
             errors.append(f"{' '.join(cmd)}\n{err}")
     if errors:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
-    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO_PATH,
+    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out,
             *[obj for _, _, obj in units]]
     if verbose:
         print(" ".join(link))
     proc = subprocess.run(link, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc link failed:\n{proc.stderr}")
-    return SO_PATH
+    return out
 
 
 class MintError(RuntimeError):

@@ -119,16 +119,30 @@ __global__ void __launch_bounds__(256) step_mix_kernel(const uint8_t* __restrict
                                                        uint8_t* staging, uint32_t staging_bytes,
                                                        uint32_t waves, uint32_t iters,
                                                        uint32_t* sink) {
+    // WHAT & 8: the own-row load writes straight into LDS (buffer_load ... lds,
+    // 16 bytes per lane) and the adder reads it from there
+    __shared__ __attribute__((aligned(16))) uint8_t landing[(WHAT & 8) ? 4 * kBlockMsg : 16];
     const LaneMap m;
     const uint32_t wave = blockIdx.x * (blockDim.x >> 6) + (uint32_t)wave_in_block();
     if (wave >= waves) return;
     const Window win(staging, staging_bytes);
     const uint32_t slot0 = wave * 2u * kBlockMsg;
+    MINT_LDS uint8_t* const mine = (MINT_LDS uint8_t*)landing +
+                                   ((WHAT & 8) ? (uint32_t)wave_in_block() * kBlockMsg : 0u);
     u32x4 acc = {0u, 0u, 0u, 0u};
     for (uint32_t i = 0; i < iters; ++i) {
         u32x4 own = {0u, 0u, 0u, 0u}, got = {0u, 0u, 0u, 0u};
         if (WHAT & 2) got = ld128<CP_SC1>(win, slot0 + (i & 1u) * kBlockMsg + m.lane * 16u);
-        if (WHAT & 1) own = ll_fetch_raw(rows, 0, i * waves + wave, true, m);
+        if constexpr ((WHAT & 9) == 9) {
+            const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
+            __builtin_amdgcn_global_load_lds(
+                (MINT_GLOBAL const void*)(rows + (uint64_t)(i * waves + wave) * kBlockRawLL + off),
+                (MINT_LDS void*)mine, 16, 0, /*nt*/ 2);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            own = *(MINT_LDS const u32x4*)(mine + m.lane * 16u);
+        } else if (WHAT & 1) {
+            own = ll_fetch_raw(rows, 0, i * waves + wave, true, m);
+        }
         const u32x4 x = add_rn<DT_F16>(own, got);
         if (WHAT & 4) st128<CP_NONE>(win, slot0 + ((i + 1u) & 1u) * kBlockMsg + m.lane * 16u, x);
         else acc ^= x;

@@ -403,7 +403,7 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
 
 int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
                   int waves, int iters, int what, void* sink, void* stream) {
-    if (waves <= 0 || iters <= 0 || what < 1 || what > 7) return MINT_ERR_ARG;
+    if (waves <= 0 || iters <= 0 || what < 1 || what > 15 || (what & 9) == 8) return MINT_ERR_ARG;
     if ((what & 1) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
         return MINT_ERR_ARG;
     if ((size_t)waves * (size_t)iters >= (1ull << 32)) return MINT_ERR_TOO_LARGE;
@@ -419,7 +419,11 @@ int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t sta
         case 4: kernel = step_mix_kernel<4>; break;
         case 5: kernel = step_mix_kernel<5>; break;
         case 6: kernel = step_mix_kernel<6>; break;
-        default: kernel = step_mix_kernel<7>; break;
+        case 7: kernel = step_mix_kernel<7>; break;
+        case 9: kernel = step_mix_kernel<9>; break;
+        case 11: kernel = step_mix_kernel<11>; break;
+        case 13: kernel = step_mix_kernel<13>; break;
+        default: kernel = step_mix_kernel<15>; break;
     }
     const unsigned blocks = ((unsigned)waves + 3u) / 4u;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, as_stream(stream),

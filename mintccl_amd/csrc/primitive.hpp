@@ -78,6 +78,7 @@ __device__ __forceinline__ void st64(const Window& w, uint32_t off, u32x2 v) {
 // count on two wait counters at once and so tie vector-memory waits to
 // scalar/LDS ones.
 #define MINT_GLOBAL __attribute__((address_space(1)))
+#define MINT_LDS __attribute__((address_space(3)))
 template <typename T>
 __device__ __forceinline__ MINT_GLOBAL T* as_global(T* p) {
     return (MINT_GLOBAL T*)p;

@@ -286,7 +286,6 @@ struct FixedRole {
 //   produced[j]   groups the fetcher has delivered     (fetcher writes)
 //   consumed[j]   groups the wave-channel has taken    (wave-channel writes)
 //   ring j        fetch_depth x U blocks of 1 KiB, arranged as ll_arrange leaves them
-#define MINT_LDS __attribute__((address_space(3)))
 constexpr uint32_t kLdsHeader = 64;       // the two counter arrays (8 wave-channels at most)
 struct LdsPort {
     MINT_LDS uint8_t* ring;
@@ -607,7 +606,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // ends on the spot instead of leaving the loop, and the prologue issues
     // exactly the queue a later step finds (stand-ins for the stores go to an
     // unused part of this wave-channel's own credit line).
+#ifdef MINT_EARLY_POLL_ALL
+    if constexpr (PROTO == PROTO_LL128) {
+#else
     if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
+#endif
       if (K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
         uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;

@@ -47,7 +47,8 @@ def step_mix(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int
              what: int = 7, sink: torch.Tensor | None = None) -> None:
     """The memory accesses of ``waves`` x ``iters`` ring steps with no ring around
     them (``what``: 1 own-row loads from ``rows``, 2 loads from ``staging``,
-    4 stores into ``staging``): the yardstick for what the device can do with
+    4 stores into ``staging``, 8 with 1: own rows loaded straight into LDS
+    instead of into registers): the yardstick for what the device can do with
     the ring kernels' mix of accesses."""
     ref = rows if rows is not None else staging
     if sink is None and not what & 4:

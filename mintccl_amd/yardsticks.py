@@ -3,7 +3,7 @@ waits for anything: ``python -m mintccl_amd.yardsticks`` prints, one JSON line
 each, the copy and read bandwidth of the library's own kernels on 1 GiB and
 the time of ``mint_step_mix`` - per wavefront and step a 960-byte own-row load
 from HBM, a 1 KiB load from and a 1 KiB store into a private staging slot, in
-every combination - for the block count of the headline launch (8 ranks x
+every combination, also with the own rows loaded straight into LDS - for the block count of the headline launch (8 ranks x
 256 MiB: 2,517,120 blocks of 1 KiB) spread over different numbers of
 wavefronts.  The ring kernels do exactly these accesses plus their flags, so
 these times are what they are measured against.  No counterpart in the
@@ -50,7 +50,9 @@ def main(argv: list[str]) -> int:
     waves_list = [int(a) for a in argv] or [1440, 2880, 3600, 4320, 5040, 5760, 7200, 11520]
     rows = torch.empty((BLOCKS + max(waves_list)) * 960, dtype=torch.uint8, device=dev).random_(0, 256)
     what = (("own rows", 1), ("staging load", 2), ("staging store", 4), ("staging load + store", 6),
-            ("own rows + staging store", 5), ("own rows + staging load", 3), ("all three", 7))
+            ("own rows + staging store", 5), ("own rows + staging load", 3), ("all three", 7),
+            ("own rows into LDS", 9), ("own rows into LDS + staging store", 13),
+            ("all three, own rows into LDS", 15))
     for waves in waves_list:
         iters = -(-BLOCKS // waves)
         staging = torch.zeros(waves * 2048, dtype=torch.uint8, device=dev)

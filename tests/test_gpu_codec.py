@@ -171,17 +171,19 @@ def test_alignment_is_rejected_not_faulted(lib, dev):
     assert lib.mint_elementwise_sum(p, p + 4, p + 2048, 8, 0, 0) == _lib.ERR_ALIGN
 
 
-def test_step_mix_moves_what_it_says(dev):
+@pytest.mark.parametrize("via_lds", [0, 8])
+def test_step_mix_moves_what_it_says(dev, via_lds):
     """The access-mix yardstick: with own-row loads and stores selected, the
     slot a wave stores into in its last step holds that step's own block in
     the lane order of the raw side (lane l, l % 4 != 3, carries the aligned
-    16-byte vector l - l // 4 of the block)."""
+    16-byte vector l - l // 4 of the block).  The same with the own rows
+    loaded straight into LDS (bit 8)."""
     from mintccl_amd import primitive
     waves, iters = 37, 5
     # f16 values in [1, 2): the store carries own + 0, which keeps such bits as they are
     rows = (torch.rand(waves * iters * 480, device=dev) + 1).to(torch.float16).view(torch.uint8)
     staging = torch.zeros(waves * 2048, dtype=torch.uint8, device=dev)
-    primitive.step_mix(rows, staging, waves, iters, what=1 | 4)
+    primitive.step_mix(rows, staging, waves, iters, what=1 | 4 | via_lds)
     torch.cuda.synchronize()
     r, s = rows.cpu().numpy(), staging.cpu().numpy()
     for w in (0, 1, 17, waves - 1):
@@ -193,8 +195,8 @@ def test_step_mix_moves_what_it_says(dev):
                 assert (slot[lane * 16: lane * 16 + 16] == block[vec * 16: vec * 16 + 16]).all()
     # all three at once only has to run; loads alone leave staging as it is
     before = staging.clone()
-    primitive.step_mix(rows, staging, waves, iters, what=1 | 2)
+    primitive.step_mix(rows, staging, waves, iters, what=1 | 2 | via_lds)
     torch.cuda.synchronize()
     assert torch.equal(staging, before)
-    primitive.step_mix(rows, staging, waves, iters, what=7)
+    primitive.step_mix(rows, staging, waves, iters, what=7 | via_lds)
     torch.cuda.synchronize()
