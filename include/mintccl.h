@@ -59,11 +59,21 @@ typedef enum {
     MINT_OP_REDUCESCATTER = 4, /* 7_reducescatter.py:13-79 */
     MINT_OP_ALLREDUCE = 5,     /* the reference's planned 8_allreduce (README.md:23):
                                   reducescatter and allgather in one pass round the ring */
-    MINT_OP_ALLTOALL = 6       /* the reference's planned 9_alltoall (README.md:24,50):
+    MINT_OP_ALLTOALL = 6,      /* the reference's planned 9_alltoall (README.md:24,50):
                                   row d of rank s goes into row s of rank d, every
                                   row straight to its destination through the
                                   destination's staging (input[] and output[] must
                                   not overlap) */
+    MINT_OP_TREE_BROADCAST = 7, /* broadcast and reduce over a binary tree, an open */
+    MINT_OP_TREE_REDUCE = 8     /* item of the reference's roadmap (README.md:52-55).
+                                  The tree is laid over ring[] turned so that the
+                                  root comes first: node h (0 = root) has parent
+                                  (h - 1) / 2 and children 2h + 1, 2h + 2.  Buffers
+                                  as for BROADCAST / REDUCE; a node's sum is
+                                  (own + first subtree) + second subtree, one
+                                  rounding per addition.  LL128 only.  slot_bytes
+                                  of a TREE_REDUCE holds two shares (one per
+                                  child). */
 } mint_op;
 typedef enum {
     MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
@@ -107,7 +117,7 @@ typedef struct {
                               (topology.py:56-93); for SENDRECV the route
                               src..dst of route_len ranks */
     int32_t route_len;     /* SENDRECV only: number of ranks on the route */
-    int32_t root;          /* BROADCAST / REDUCE root rank */
+    int32_t root;          /* BROADCAST / REDUCE / TREE_* root rank */
     uint64_t input[MINT_MAX_RANKS];   /* per rank; 0 = absent */
     uint64_t output[MINT_MAX_RANKS];  /* per rank; 0 = absent */
     uint64_t staging[MINT_MAX_RANKS]; /* per rank, mint_ring_staging_bytes() each */
@@ -116,7 +126,7 @@ typedef struct {
                               fit is refused with MINT_ERR_STAGING (the credit
                               words sit behind the slots, outside a buffer
                               that only holds nslots * slot_bytes) */
-    uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE: bytes of the
+    uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE/TREE_*: bytes of the
                               buffer; ALLGATHER/REDUCESCATTER/ALLTOALL: bytes of
                               one row */
     uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER/ALLTOALL: bytes between rows */
@@ -241,7 +251,8 @@ int mint_ring_grid_blocks(const mint_ring_op* op);
  * 1024 for Simple), recv_offset[i] / send_offset[i] (byte offset of the
  * block's 1 KiB message inside the staging of the rank it is received in /
  * sent to).  Any output array may be NULL; at most max_entries are written,
- * *n_entries is the full count.  Needs no GPU. */
+ * *n_entries is the full count.  Needs no GPU.  The tree ops are not listed
+ * (MINT_ERR_ARG). */
 int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
                        uint32_t max_entries, uint32_t* step, uint32_t* block,
                        uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries);

@@ -1,5 +1,6 @@
 """Ring broadcast (``4_broadcast.py``): after the call every rank's ``buff``
-holds the root's bytes."""
+holds the root's bytes.  ``MINTCCL_TOPOLOGY=tree`` sends them down a binary tree
+instead (``mintccl_amd.tree``)."""
 from __future__ import annotations
 
 import torch
@@ -10,6 +11,9 @@ from .common import VirtualComm
 
 
 def broadcast(buff: torch.Tensor, root: int, comm: VirtualComm | None = None) -> None:
+    from . import tree
+    if tree.topology_env() == "tree":
+        return tree.broadcast(buff, root, comm)
     comm = comm_or_default(comm)
     check_buffer(buff, comm)
     posted = comm.post("broadcast", set(range(comm.world_size)),

@@ -153,6 +153,13 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         granule = wpb * (8 // math.gcd(world * world, 8))      # whole channels for every XCD
         waves = max(granule, total // (2 * world * world) // granule * granule)
         return world * waves * 1024, min(max_nslots, TUNED_NSLOTS_MULTI), waves
+    if op in (_lib.OP_TREE_BROADCAST, _lib.OP_TREE_REDUCE):
+        # one wavefront per (node, wave-channel); a reducing node's slot has a
+        # share per child
+        shares = 2 if op == _lib.OP_TREE_REDUCE else 1
+        granule = max(1, threads_per_block // 64) * 8
+        waves = max(granule, min(TUNED_SLOT_BLOCKS, TUNED_TOTAL_WAVES // world) // granule * granule)
+        return shares * waves * 1024, max_nslots, waves
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
     real_pipes = pipes
     if op == _lib.OP_ALLREDUCE:
@@ -363,6 +370,9 @@ class VirtualComm:
                                           _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL) else 1
         if op == _lib.OP_ALLREDUCE:
             pipes *= 2            # a slot is shared by (pipeline, phase): two phases
+        tree = op in (_lib.OP_TREE_BROADCAST, _lib.OP_TREE_REDUCE)
+        if op == _lib.OP_TREE_REDUCE:
+            pipes = 2             # a slot has a share per child
         threads = self.threads_per_block
         reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
         if self.auto_geometry:
@@ -380,7 +390,7 @@ class VirtualComm:
                     "slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
             # (an alltoall has twice `pipes` groups of wave-channels per rank: it
             # sends `world` rows and receives `world` rows)
-            groups = 2 * pipes if op == _lib.OP_ALLTOALL else pipes
+            groups = 2 * pipes if op == _lib.OP_ALLTOALL else (1 if tree else pipes)
             d.waves_per_channel_group = _largest_divisor_at_most(
                 step_blocks, max(1, self.waves_per_rank // groups))
         d.threads_per_block = threads
@@ -393,6 +403,8 @@ class VirtualComm:
             real_pipes = pipes // 2 if op == _lib.OP_ALLREDUCE else pipes
             if op == _lib.OP_ALLTOALL:
                 real_pipes = self.world_size * self.world_size
+            if tree:
+                real_pipes = 1
             channels = real_pipes * -(-d.waves_per_channel_group // wpb)
             if channels % 8:
                 d.placement = _lib.PLACE_SPREAD

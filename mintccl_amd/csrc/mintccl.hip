@@ -7,6 +7,7 @@
 
 #include "kernels.hpp"
 #include "ring_launch.hpp"
+#include "tree.hpp"
 
 using namespace mint;
 
@@ -32,8 +33,12 @@ inline bool aligned16(uint64_t p) { return (p & 15u) == 0; }
 inline bool aligned16(const void* p) { return aligned16(reinterpret_cast<uint64_t>(p)); }
 
 bool reducing(int op) {
-    return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE;
+    return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE ||
+           op == MINT_OP_TREE_REDUCE;
 }
+bool over_tree(int op) { return op == MINT_OP_TREE_BROADCAST || op == MINT_OP_TREE_REDUCE; }
+static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE == OP_TREE_REDUCE,
+              "op codes");
 
 // Everything the launch derives from the descriptor.  `for_launch`: also
 // check what only matters once the kernels run (the size of the staging the
@@ -41,9 +46,11 @@ bool reducing(int op) {
 int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
               const mint_ring_debug* dbg = nullptr) {
     if (!op || !plan) return MINT_ERR_ARG;
-    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLTOALL) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_TREE_REDUCE) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
+    // the tree kernels speak LL128 only
+    if (over_tree(op->op) && op->protocol != MINT_PROTO_LL128) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
     if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
     if (op->cache_policy < 0 || op->cache_policy > 2) return MINT_ERR_ARG;
@@ -75,6 +82,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // a rank receives from every pipeline that passes through it: one share of
     // its slots per pipeline and phase; in an alltoall, one per source rank
     a.shares = alltoall ? op->world : a.pipes * a.phases;
+    // a node of a reducing tree receives from two children: a share of its slots each
+    if (op->op == MINT_OP_TREE_REDUCE) a.shares = kTreeArity;
 
     // ring / route
     bool seen[MINT_MAX_RANKS] = {};
@@ -100,9 +109,12 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     switch (op->op) {
         case MINT_OP_SENDRECV:  a.hops = a.cyc_len - 1; a.start[0] = 0; break;
         case MINT_OP_BROADCAST:
-        case MINT_OP_REDUCE: {
+        case MINT_OP_REDUCE:
+        case MINT_OP_TREE_BROADCAST:
+        case MINT_OP_TREE_REDUCE: {
             if (op->root < 0 || op->root >= op->world) return MINT_ERR_ARG;
-            a.hops = op->op == MINT_OP_BROADCAST ? op->world - 1 : op->world;
+            // (a tree has one position per node)
+            a.hops = op->op == MINT_OP_REDUCE ? op->world : op->world - 1;
             a.start[0] = (uint8_t)index_of(op->root);
             break;
         }
@@ -140,7 +152,16 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
                   (op->op == MINT_OP_SENDRECV && a.cyc_len == 1);
 
     // which ranks need which buffers
-    for (int p = 0; p < a.pipes && !plan->empty; ++p) {
+    for (int h = 0; h < op->world && over_tree(op->op) && !plan->empty; ++h) {
+        const int rank = tree_rank(a, h);
+        const bool up = op->op == MINT_OP_TREE_REDUCE;
+        const bool receives = up ? tree_children(h, op->world) > 0 : h != 0;
+        if ((up || h == 0) && !op->input[rank]) return MINT_ERR_ARG;
+        if ((up ? h == 0 : h != 0) && !op->output[rank]) return MINT_ERR_ARG;
+        if (receives && (!op->staging[rank] || !aligned16(op->staging[rank])))
+            return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+    }
+    for (int p = 0; p < a.pipes && !plan->empty && !over_tree(op->op); ++p) {
         for (int h = 0; h <= a.hops; ++h) {
             const int rank = alltoall ? (h == 0 ? p / op->world : p % op->world)
                                       : a.cyc[(a.start[p] + h) % a.cyc_len];
@@ -214,7 +235,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // step.  Everything else runs the walk that fetches its rows itself.
     a.k_per_wave = a.step_blocks / (uint32_t)a.waves;
     plan->lds = op->row_fetch == MINT_FETCH_LDS && op->protocol == MINT_PROTO_LL128 &&
-                reducing(op->op) && (waves_per_block == 4 || waves_per_block == 7) &&
+                reducing(op->op) && !over_tree(op->op) &&
+                (waves_per_block == 4 || waves_per_block == 7) &&
                 a.k_per_wave % 4 != 0;
     a.fetch_depth = plan->lds ? kFetchDepth : 0u;
     if (!plan->lds && a.waves < waves_per_block) plan->threads = a.waves * 64;
@@ -544,6 +566,7 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
     const int err = make_plan(op, &plan);
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
+    if (over_tree(op->op)) return MINT_ERR_ARG;     // listed for the ring walks only
     const RingArgs& a = plan.args;
     if (pipeline < 0 || pipeline >= a.pipes || position < 0 || position > a.hops || wave < 0 ||
         wave >= a.waves)

@@ -3,6 +3,7 @@
 #include <atomic>
 
 #include "ring_launch.hpp"
+#include "tree.hpp"
 
 #ifndef MINT_FAMILY_DT
 #error "compile with -DMINT_FAMILY_DT=0..3"
@@ -107,8 +108,37 @@ int launch_ring_cp(const Plan& plan, int cache_policy, hipStream_t stream) {
     }
 }
 
+// Broadcast / reduce over a binary tree (LL128): one wavefront per (node,
+// wave-channel), all of them resident like a ring's.
+template <int DT, int CP>
+int launch_tree(const Plan& plan, hipStream_t stream) {
+    void (*kernel)(const RingArgs) = tree_kernel<DT, CP>;
+    static std::atomic<int> cached[9] = {};          // [threads / 64]
+    static std::atomic<int> cus{0};
+    std::atomic<int>& memo = cached[plan.threads / 64];
+    int per_cu = memo.load(std::memory_order_relaxed);
+    if (per_cu == 0) {
+        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
+        if (per_cu < 0) return MINT_ERR_HIP;
+        memo.store(per_cu, std::memory_order_relaxed);
+    }
+    int ncu = cus.load(std::memory_order_relaxed);
+    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
+    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
+                       plan.args);
+    return launch_status();
+}
+
 template <int DT>
 int launch_family(const Plan& plan, int protocol, int cache_policy, hipStream_t stream) {
+    if (plan.args.op == OP_TREE_BROADCAST || plan.args.op == OP_TREE_REDUCE) {
+        switch (cache_policy) {
+            case 0: return launch_tree<DT, 0>(plan, stream);
+            case 1: return launch_tree<DT, 1>(plan, stream);
+            default: return launch_tree<DT, 2>(plan, stream);
+        }
+    }
     return protocol == MINT_PROTO_LL128 ? launch_ring_cp<PROTO_LL128, DT>(plan, cache_policy, stream)
                                         : launch_ring_cp<PROTO_SIMPLE, DT>(plan, cache_policy, stream);
 }

@@ -1,0 +1,174 @@
+// Broadcast and reduce over a binary tree of the virtual ranks.
+//
+// Reference: none yet - "Tree / Binary Tree" is an open item of the
+// reference's roadmap (README.md:52-55).  The pieces are the reference's:
+// load / recv / comp / save / send of LL128 blocks in the order of
+// 4_broadcast.py:55-70 and 5_reduce.py:70-89, through circular staging slots
+// with a credit word per edge (protocol.py:161-189).
+//
+// The tree is laid over the ring order the launch names, turned so that the
+// root comes first: node h (0 = root) is rank cyc[(start + h) % world], its
+// parent is node (h - 1) / 2, its children are nodes 2h + 1 and 2h + 2 where
+// they exist.  Eight ranks are three hops deep where the ring is seven.
+//
+//   broadcast  a node takes a block from its parent's send (the root: from
+//              its own buffer), keeps a copy (all but the root) and sends it
+//              to both children
+//   reduce     a node adds to its own block the block of its first child,
+//              then that of its second child, one rounding each, and sends
+//              the sum to its parent (the root: stores it)
+//
+// so the value a node passes up is  (own + first subtree) + second subtree.
+//
+// One wavefront serves one (node, wave-channel) and does everything that node
+// does with the wave-channel's blocks; wave-channel w of a node talks only to
+// wave-channel w of its parent and children, as on the ring.  A node that
+// receives from two children has two shares in each of its slots, one per
+// child, and a credit word for each.
+#pragma once
+#include "ring.hpp"
+
+namespace mint {
+
+enum : int { OP_TREE_BROADCAST = 7, OP_TREE_REDUCE = 8 };
+constexpr int kTreeArity = 2;
+
+__host__ __device__ __forceinline__ int tree_rank(const RingArgs& a, int h) {
+    return a.cyc[(a.start[0] + h) % a.world];
+}
+__host__ __device__ __forceinline__ int tree_children(int h, int world) {
+    const int c = world - (kTreeArity * h + 1);
+    return c < 0 ? 0 : (c > kTreeArity ? kTreeArity : c);
+}
+
+template <int DT, int CPI>
+__device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const int w) {
+    constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;
+    const LaneMap m;
+    const bool reduce = a.op == OP_TREE_REDUCE;
+    const int rank = tree_rank(a, h);
+    const int nchild = tree_children(h, a.world);
+    // data flows down the tree in a broadcast, up in a reduce
+    const int nin = reduce ? nchild : (h ? 1 : 0);
+    const int nout = reduce ? (h ? 1 : 0) : nchild;
+    const bool load = reduce || h == 0;
+    const bool save = reduce ? h == 0 : h != 0;
+
+    const uint64_t row_bytes = a.row_bytes;
+    const uint32_t nblocks = a.nblocks;
+    const uint8_t* in_row = reinterpret_cast<const uint8_t*>(a.input[rank]);
+    uint8_t* out_row = reinterpret_cast<uint8_t*>(a.output[rank]);
+    const uint32_t ring_bytes = a.nslots * a.slot_bytes;
+    const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
+
+    // where this node sends: rank, and which share of that rank's slots
+    int to[kTreeArity];
+    uint32_t to_share[kTreeArity];
+#pragma unroll
+    for (int j = 0; j < kTreeArity; ++j) {
+        if (reduce) {
+            to[j] = h ? tree_rank(a, (h - 1) / kTreeArity) : rank;
+            to_share[j] = h ? (uint32_t)((h - 1) % kTreeArity) : 0u;
+        } else {
+            to[j] = j < nchild ? tree_rank(a, kTreeArity * h + 1 + j) : rank;
+            to_share[j] = 0u;
+        }
+    }
+    const Window own(reinterpret_cast<const void*>(a.staging[rank]), ring_bytes);
+    const Window out0(reinterpret_cast<const void*>(a.staging[to[0]]), ring_bytes);
+    const Window out1(reinterpret_cast<const void*>(a.staging[to[1]]), ring_bytes);
+    auto credit_word = [&](int of_rank, uint32_t share) {
+        return reinterpret_cast<uint64_t*>(a.staging[of_rank] + a.credit_off +
+                                           (share * W + (uint32_t)w) * kCreditStride);
+    };
+    uint64_t* const in_tail[kTreeArity] = {credit_word(rank, 0u), credit_word(rank, 1u)};
+    const uint64_t* const out_tail[kTreeArity] = {credit_word(to[0], to_share[0]),
+                                                  credit_word(to[1], to_share[1])};
+
+    const uint32_t epoch =
+        a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
+                           as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                     : a.epoch;
+    const uint64_t flag_hi = (uint64_t)epoch << 32;
+    uint32_t credits_seen[kTreeArity] = {0u, 0u};
+
+    uint32_t slot = 0;
+    for (uint32_t s = 0; s < a.steps; ++s) {
+        const uint32_t tag = (epoch << 20) | (s + 1u);
+        // wait_ll128 (protocol.py:161-180): the receiver has emptied the slot
+        // this step goes into
+        const uint32_t need = s >= a.nslots ? s - a.nslots + 1 : 0;
+#pragma unroll
+        for (int j = 0; j < kTreeArity; ++j)
+            if (j < nout && !wait_count(out_tail[j], epoch, need, credits_seen[j], a.spin_budget,
+                                        a.status)) {
+                report_timeout(a.status, 0, h, w, s);
+                return;
+            }
+        for (uint32_t k = 0; k < K; ++k) {
+            const uint32_t idx = k * W + (uint32_t)w;
+            const uint32_t g = s * a.step_blocks + idx;
+            if (g >= nblocks) break;
+            const uint32_t at = slot * a.slot_bytes + idx * kBlockMsg;
+            u32x4 x = {0u, 0u, 0u, 0u};
+            if (load) x = ll_load_raw(in_row, row_bytes, g, m);
+            // first poll of every incoming block at once, then the repeats
+            u32x4 r[kTreeArity];
+            uint32_t pending = 0;
+            compiler_fence();
+#pragma unroll
+            for (int j = 0; j < kTreeArity; ++j)
+                if (j < nin && !ll_poll<LDCP>(own, at + (uint32_t)j * a.step_msg, tag, m, r[j]))
+                    pending |= 1u << j;
+            for (uint32_t spins = 0; pending; ++spins) {
+                if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
+                    report_timeout(a.status, 0, h, w, s);
+                    return;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                compiler_fence();
+#pragma unroll
+                for (int j = 0; j < kTreeArity; ++j)
+                    if ((pending & (1u << j)) &&
+                        ll_poll<LDCP>(own, at + (uint32_t)j * a.step_msg, tag, m, r[j]))
+                        pending &= ~(1u << j);
+            }
+#pragma unroll
+            for (int j = 0; j < kTreeArity; ++j) {
+                if (j >= nin) continue;
+                if constexpr (DT != DT_BYTES) {
+                    x = reduce ? ll_comp<DT>(x, r[j]) : r[j];
+                } else {
+                    x = r[j];
+                }
+            }
+            if (save) ll_save_raw(out_row, row_bytes, g, m, x);
+            if (nout > 0) ll_send<STCP>(out0, at + to_share[0] * a.step_msg, x, tag, m);
+            if (nout > 1) ll_send<STCP>(out1, at + to_share[1] * a.step_msg, x, tag, m);
+        }
+        // post_ll128 (protocol.py:183-189): every block of step s has been
+        // taken out of this node's slot (the polls tested what they loaded)
+        if (lane_id() == 0) {
+#pragma unroll
+            for (int j = 0; j < kTreeArity; ++j) {
+                if (j >= nin) continue;
+                if (STCP == CP_NONE) st64_local(in_tail[j], flag_hi | (uint64_t)(s + 1));
+                else st64_agent(in_tail[j], flag_hi | (uint64_t)(s + 1));
+            }
+        }
+        slot = slot + 1 == a.nslots ? 0 : slot + 1;
+    }
+}
+
+// Seats are dealt as for the ring kernels (position = node of the tree), so
+// with the local placement a wave-channel's whole tree shares one XCD.
+template <int DT, int CPI>
+__global__ void __launch_bounds__(512) tree_kernel(const RingArgs a) {
+    const int wpb = (int)(blockDim.x >> 6);
+    const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
+    const Seat st = take_seat(a, wpb, wib);
+    if (!st.ok) return;
+    tree_walk<DT, CPI>(a, st.h, st.w);
+}
+
+}  // namespace mint

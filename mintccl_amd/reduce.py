@@ -1,5 +1,6 @@
 """Ring reduce (``5_reduce.py``): elementwise sum in ring order, in place at
-the root; the other ranks' buffers are left as they were."""
+the root; the other ranks' buffers are left as they were.
+``MINTCCL_TOPOLOGY=tree`` adds up a binary tree instead (``mintccl_amd.tree``)."""
 from __future__ import annotations
 
 import torch
@@ -11,6 +12,9 @@ from .common import VirtualComm
 
 
 def reduce(buff: torch.Tensor, root: int, comm: VirtualComm | None = None) -> None:
+    from . import tree
+    if tree.topology_env() == "tree":
+        return tree.reduce(buff, root, comm)
     comm = comm_or_default(comm)
     check_buffer(buff, comm)
     posted = comm.post("reduce", set(range(comm.world_size)),

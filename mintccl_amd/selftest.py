@@ -233,13 +233,55 @@ def alltoall() -> bool:
                 for d in range(world)])
 
 
+def _tree_fold(rows: list[torch.Tensor], order: list[int], h: int = 0) -> torch.Tensor:
+    """(own + first subtree) + second subtree, node ``h`` of the tree over ``order``."""
+    acc = rows[order[h]].clone()
+    for c in (2 * h + 1, 2 * h + 2):
+        if c < len(order):
+            acc = acc + _tree_fold(rows, order, c)
+    return acc
+
+
+def tree_broadcast() -> bool:
+    """What 4_broadcast.py:104-126 checks, down the binary tree (README.md:52-55)."""
+    from .tree import broadcast as op
+    comm = VirtualComm()
+    dev, n, root = comm.device, common.test_count(), _env_rank("ROOT_TEMP", 0)
+    g = _gen(dev)
+    bufs = [torch.randn(n, device=dev, generator=g) if r == root else torch.empty(n, device=dev)
+            for r in range(comm.world_size)]
+    want = bufs[root].clone()
+    _run_all(comm, lambda r: op(bufs[r], root, comm))
+    if not common.test_mode():
+        return True
+    return all([_report(r, bufs[r], want, r == (root + 1) % comm.world_size)
+                for r in range(comm.world_size)])
+
+
+def tree_reduce() -> bool:
+    """What 5_reduce.py:123-155 checks, up the binary tree (README.md:52-55)."""
+    from ._ops import ring_of
+    from .tree import nodes, reduce as op
+    comm = VirtualComm()
+    root = _env_rank("ROOT_TEMP", 0)
+    bufs = _reduction_inputs(comm, (common.test_count(),))
+    inputs = [b.clone() for b in bufs] if common.test_mode() else None
+    _run_all(comm, lambda r: op(bufs[r], root, comm))
+    if inputs is None:
+        return True
+    want = _tree_fold(inputs, nodes(ring_of(comm), root))
+    _order_free_distance(root, bufs[root], inputs)
+    return _report(root, bufs[root], want, True)
+
+
 def main(name: str) -> int:
     from . import sendrecv_buffer, sendrecv_indirect
     tests = {"sendrecv_direct": sendrecv_direct,
              "sendrecv_indirect": lambda: sendrecv(sendrecv_indirect),
              "sendrecv_buffer": lambda: sendrecv(sendrecv_buffer),
              "broadcast": broadcast, "reduce": reduce, "allgather": allgather,
-             "reducescatter": reducescatter, "allreduce": allreduce, "alltoall": alltoall}
+             "reducescatter": reducescatter, "allreduce": allreduce, "alltoall": alltoall,
+             "tree_broadcast": tree_broadcast, "tree_reduce": tree_reduce}
     if name == "all":
         return 0 if all([fn() for fn in tests.values()]) else 1
     return 0 if tests[name]() else 1

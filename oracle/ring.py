@@ -191,6 +191,37 @@ def broadcast(xs: list, root: int) -> list:
     return [_bytes(xs[root]).copy() for _ in xs]
 
 
+def tree_nodes(ring: list[int], root: int) -> list[int]:
+    """Ranks in node order of the binary tree laid over the ring turned to the
+    root: node h has parent (h - 1) // 2 and children 2h + 1, 2h + 2."""
+    return fold_order(ring, root)
+
+
+def tree_fold(rows: list, nodes: list[int], dtype: str, h: int = 0) -> np.ndarray:
+    """What node h passes to its parent: (own + first subtree) + second
+    subtree, one rounding per addition."""
+    acc = _bytes(rows[nodes[h]]).copy()
+    for c in (2 * h + 1, 2 * h + 2):
+        if c < len(nodes):
+            acc = add_rn(acc, tree_fold(rows, nodes, dtype, c), dtype)
+    return acc
+
+
+def tree_reduce(xs: list, root: int, dtype: str, ring: list[int] | None = None) -> list:
+    """Reduce up a binary tree ("Tree / Binary Tree" is an open item of the
+    reference's roadmap, ``README.md:52-55``; the reference holds no code for
+    it, so the order of the additions is this build's definition - parity with
+    the reference is unpinned by construction).  The building blocks are the
+    reference's: ``comp_ll128`` (``protocol.py:142-156``) adds own + received
+    with one rounding.  Pinned: against hand-computed values that tell this
+    order from the ring's and from (first + second) + own; equal to
+    ``reduce`` for N = 2; within (N - 1) half-ulp steps of the exact sum."""
+    ring = ring or identity_ring(len(xs))
+    out = [_bytes(x).copy() for x in xs]
+    out[root] = tree_fold(xs, tree_nodes(ring, root), dtype)
+    return out
+
+
 def sendrecv(xs: list, src: int, dst: int) -> list:
     out = [_bytes(x).copy() for x in xs]
     out[dst] = _bytes(xs[src]).copy()

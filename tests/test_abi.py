@@ -131,7 +131,10 @@ def test_plan_geometry_without_a_gpu():
 
 @pytest.mark.parametrize("kw,err", [
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
-    (dict(op=7), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=9), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=_lib.OP_TREE_REDUCE, protocol=_lib.PROTO_SIMPLE, waves_per_channel_group=128),
+     _lib.ERR_ARG),                                      # the tree kernels speak LL128 only
+    (dict(op=_lib.OP_TREE_REDUCE, dtype=_lib.BYTES, waves_per_channel_group=128), _lib.ERR_ARG),
     (dict(dtype=_lib.BYTES), _lib.ERR_ARG),          # a reduction needs a real dtype
     (dict(flag_epoch=0), _lib.ERR_ARG), (dict(flag_epoch=4096), _lib.ERR_ARG),
     (dict(status=0), _lib.ERR_ARG), (dict(cache_policy=3), _lib.ERR_ARG),
@@ -178,6 +181,45 @@ def test_plan_rejects_bad_buffers_and_rings():
     d = make_op()
     d.ring[3] = 2                                    # rank 2 twice
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+
+
+def test_tree_plans_without_a_gpu():
+    """Broadcast / reduce over a binary tree: one position per node; a reducing
+    node's slot holds a share per child, with a credit word each."""
+    L = _lib.lib()
+    d = make_op(op=_lib.OP_TREE_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256
+    d = make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=128, root=3)
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 2 * 128 * 256
+    # 512 KiB slot / 2 shares = 256 blocks per step
+    assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=512)) \
+        == _lib.ERR_GEOMETRY
+    # buffers: root 3 heads the node order 3, 4, 5, 6, 7, 0, 1, 2; nodes 4..7 of it
+    # (ranks 7, 0, 1, 2) are leaves and receive nothing in a reduce
+    d = make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=128, root=3)
+    for leaf in (7, 0, 1, 2):
+        d.staging[leaf] = 0
+    for r in range(8):
+        if r != 3:
+            d.output[r] = 0
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    d.staging[4] = 0                                 # node 1 has children
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+    d = make_op(op=_lib.OP_TREE_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
+    d.staging[3] = 0                                 # the root of a broadcast receives nothing
+    for r in range(8):
+        if r != 3:
+            d.input[r] = 0
+    d.output[3] = 0
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    d.output[5] = 0
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+    # the schedule listing covers the ring walks only
+    n = ctypes.c_uint32(0)
+    d = make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=128)
+    assert L.mint_ring_schedule(d, 0, 0, 0, 0, None, None, None, None, ctypes.byref(n)) == _lib.ERR_ARG
 
 
 def test_launch_refuses_undersized_staging_before_touching_the_gpu():

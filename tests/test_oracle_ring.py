@@ -122,6 +122,51 @@ def test_reduce_order_follows_ring_from_root():
                 assert (out[r] == xs[r]).all()       # non-roots keep their data
 
 
+def test_hand_computed_tree_order():
+    """Binary tree over the node order: (own + first subtree) + second subtree."""
+    f = lambda *v: [np.array([x], dtype=np.float16).view(np.uint8) for x in v]
+    as_f = lambda raw: float(raw.view(np.float16)[0])
+    # three nodes: (2048 + 1) + 1 = 2048 where (1 + 1) + 2048 would give 2050
+    assert as_f(ring.tree_fold(f(2048.0, 1.0, 1.0), [0, 1, 2], "f16")) == 2048.0
+    # first child before second: (2048 + 1) -> 2048, + 1.5 -> 2050;
+    # the other way round (2048 + 1.5) -> 2050, + 1 = 2051 -> 2052
+    assert as_f(ring.tree_fold(f(2048.0, 1.0, 1.5), [0, 1, 2], "f16")) == 2050.0
+    assert as_f(ring.tree_fold(f(2048.0, 1.5, 1.0), [0, 1, 2], "f16")) == 2052.0
+    # five nodes: node 1 has children 3 and 4.  Tree: (2048 + ((1 + 1) + 0)) + 0 = 2050;
+    # the ring order ((((2048 + 1) + 0) + 1) + 0) loses both ones: 2048
+    rows = f(2048.0, 1.0, 0.0, 1.0, 0.0)
+    assert as_f(ring.tree_fold(rows, [0, 1, 2, 3, 4], "f16")) == 2050.0
+    assert as_f(ring.fold(rows, [0, 1, 2, 3, 4], "f16")) == 2048.0
+    # the node order is the ring turned to the root
+    assert ring.tree_nodes([0, 2, 1, 3, 4, 0], 1) == [1, 3, 4, 0, 2]
+    xs = [rows[i] for i in (3, 0, 4, 1, 2)]        # rank r holds the value of node [1,3,4,0,2].index(r)
+    out = ring.tree_reduce(xs, 1, "f16", [0, 2, 1, 3, 4, 0])
+    assert as_f(out[1]) == 2050.0
+    assert all((out[r] == xs[r]).all() for r in (0, 2, 3, 4))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_tree_reduce_properties(dt):
+    bits = 32 if dt == "f32" else 16
+    # two ranks: one commutative addition, the same as the ring's
+    a, b = random_bits(4000, bits, 31), random_bits(4000, bits, 32)
+    x = [a.view(np.uint8), b.view(np.uint8)]
+    assert ring.same_values(ring.tree_reduce(x, 1, dt)[1], ring.reduce(x, 1, dt)[1], dt)
+    # small integers add exactly in any order: the tree and the ring agree with the plain sum
+    rng = np.random.default_rng(5)
+    vals = [rng.integers(-8, 9, 1000).astype(np.float32) for _ in range(7)]
+    if dt == "f32":
+        raw = [v.view(np.uint8) for v in vals]
+    elif dt == "f16":
+        raw = [v.astype(np.float16).view(np.uint8) for v in vals]
+    else:
+        raw = [(v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8) for v in vals]
+    for root in (0, 3, 6):
+        t = ring.tree_reduce(raw, root, dt)[root]
+        assert ring.same_values(t, ring.reduce(raw, root, dt)[root], dt)
+        assert np.array_equal(ring.to_float64(t, dt), np.sum(vals, axis=0, dtype=np.float64))
+
+
 def test_fold_order_with_a_permuted_ring():
     ring_ = [0, 2, 1, 3, 0]
     assert ring.fold_order(ring_, 1) == [1, 3, 0, 2]
