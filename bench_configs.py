@@ -244,6 +244,27 @@ def config5(reps: int, max_log2: int) -> None:
                      shard_bytes=shard, us=round(ms * 1e3, 2),
                      alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1), hbm_bytes=world * S,
                      busbw_gbps=round(shard * (world - 1) / ms / 1e6, 1), ok=ok)
+                if label == "tuned" and log2 <= 16 and log2 % 2 == 1:
+                    # the same launch as 20 nodes of a HIP graph (epoch in device
+                    # memory, advanced by a small kernel in front of every launch):
+                    # what the device needs once the host is out of the way
+                    gcomm = VirtualComm(world_size=world, device=DEV, protocol=proto,
+                                        device_epoch=True)
+                    gd = gcomm.make_op(_lib.OP_ALLGATHER, _lib.BYTES, shard, ptrs, ptrs,
+                                       list(range(world)) + [0], row_stride=shard)
+                    side = torch.cuda.Stream(device=DEV)
+                    with torch.cuda.stream(side):
+                        gcomm.launch(gd)
+                    side.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        for _ in range(20):
+                            gcomm.launch(gd)
+                    gms = time_ms(graph.replay, reps * 2) / 20
+                    gcomm.check()
+                    gok = all(torch.equal(b.view(torch.int16), want.view(torch.int16)) for b in bufs)
+                    emit(config=5, op="allgather", protocol=name, staging="tuned, graph of 20",
+                         world=world, shard_bytes=shard, us=round(gms * 1e3, 2), ok=gok)
             del bufs
 
 
@@ -324,12 +345,68 @@ def alltoall_bench(reps: int) -> None:
         del bufs, outs
 
 
+def tree_bench(reps: int, log2s=(10, 14, 17, 20, 23, 26)) -> None:
+    """Broadcast and reduce over the binary tree (3 hops deep for 8 ranks)
+    beside the ring (7 / 8 hops), 8 ranks, from 1 KiB to 64 MiB per rank,
+    launched from prepared descriptors; checked against the device adder folded
+    in the tree's / the ring's order."""
+    from mintccl_amd import primitive
+    world, root = 8, 0
+    comm = comm_for(world, 0)
+    ring = list(range(world)) + [0]
+    for log2 in log2s:
+        nbytes = 1 << log2
+        n = nbytes // 2
+        g = torch.Generator(device=DEV).manual_seed(9)
+        src = [(torch.rand(n, generator=g, device=DEV) * 2 - 1).to(torch.float16) for _ in range(world)]
+
+        def tree_sum(h: int) -> torch.Tensor:
+            acc = src[h].clone()
+            for c in (2 * h + 1, 2 * h + 2):
+                if c < world:
+                    acc = primitive.Sum(acc, tree_sum(c))
+            return acc
+
+        want = {"tree": tree_sum(0), "ring": fold_device(src, list(range(world)))}
+        bufs = [x.clone() for x in src]
+        ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+        for topo, rd, bc in (("ring", _lib.OP_REDUCE, _lib.OP_BROADCAST),
+                             ("tree", _lib.OP_TREE_REDUCE, _lib.OP_TREE_BROADCAST)):
+            for b, x in zip(bufs, src):
+                b.copy_(x)
+            d = comm.make_op(rd, _lib.F16, nbytes, ptrs, {root: ptrs[root]}, ring, root=root,
+                             protocol=_lib.PROTO_LL128)
+            comm.launch(d)
+            comm.check()
+            ok = torch.equal(bufs[root], want[topo]) and all(
+                torch.equal(bufs[r], src[r]) for r in range(1, world))
+            # (timed launches keep adding into the root's buffer: the values no longer matter)
+            ms = time_ms(lambda: comm.launch(d), reps * 4)
+            comm.check()
+            emit(config="tree", op="reduce", topology=topo, world=world, bytes=nbytes,
+                 us=round(ms * 1e3, 2), hbm_bytes=(world + 1) * nbytes, ok=ok, grid=comm.last_grid)
+            d = comm.make_op(bc, _lib.BYTES, nbytes, {root: ptrs[root]},
+                             {r: p for r, p in ptrs.items() if r != root}, ring, root=root,
+                             protocol=_lib.PROTO_LL128)
+            for b in bufs[1:]:
+                b.zero_()
+            comm.launch(d)
+            comm.check()
+            ok = all(torch.equal(b, bufs[root]) for b in bufs)
+            ms = time_ms(lambda: comm.launch(d), reps * 4)
+            comm.check()
+            emit(config="tree", op="broadcast", topology=topo, world=world, bytes=nbytes,
+                 us=round(ms * 1e3, 2), hbm_bytes=world * nbytes, ok=ok, grid=comm.last_grid)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--staging", choices=("both", "reference", "tuned"), default="both")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
     ap.add_argument("--only", type=int, default=0,
-                    help="run one config (2..5; 8 = allreduce; 9 = alltoall)")
+                    help="run one config (2..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring)")
+    ap.add_argument("--tree-log2", default="10,14,17,20,23,26",
+                    help="config 10: log2 of the message sizes (bytes per rank)")
     args = ap.parse_args()
     global STAGING
     STAGING = ("reference", "tuned") if args.staging == "both" else (args.staging,)
@@ -347,6 +424,8 @@ def main() -> int:
         allreduce_bench(reps)
     if args.only in (0, 9):
         alltoall_bench(reps)
+    if args.only in (0, 10):
+        tree_bench(reps, tuple(int(x) for x in args.tree_log2.split(",")))
     return 0
 
 

@@ -67,3 +67,11 @@ def test_headline_geometry():
     assert common.tuned_geometry(_lib.OP_ALLREDUCE, 8, 0, 128, 3) == (512 * 1024, 3, 32)
     assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
+    # a small message takes a small grid: the wave-channels are capped at the
+    # blocks of one row, in whole thread blocks that the 8 XCDs divide
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=1) == (32 * 1024, 2, 4)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=69) == (576 * 1024, 2, 72)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=10 ** 6) == (640 * 1024, 2, 80)
+    assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3, row_blocks=5) == (32 * 1024, 3, 32)
+    assert common.tuned_geometry(_lib.OP_TREE_REDUCE, 8, 0, 256, 3, row_blocks=5) == (2 * 32 * 1024, 3, 32)
+    assert common.tuned_geometry(_lib.OP_TREE_REDUCE, 8, 0, 256, 3) == (2 * 512 * 1024, 3, 512)
