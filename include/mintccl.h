@@ -102,6 +102,12 @@ typedef enum {
  * that gave up; word 2: step it waited for; word 3: abort flag polled by all
  * other waits.  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
  * then holds that number.
+ * The words stay set until the caller zeroes them: every launch that finds
+ * word 3 set gives up at its first wait (after at most 64 polls) and leaves
+ * unspecified output, and only the first failure is recorded.  After a
+ * non-zero word 0 the caller synchronises the stream, zeroes the block (the
+ * staging needs no clearing: the next launch brings its own epoch) and treats
+ * the outputs of every launch since the last clean check as lost.
  * The reference has no abort path (common.py:106 is unused). */
 #define MINT_STATUS_WORDS 4
 
@@ -177,7 +183,14 @@ const char* mint_strerror(int err);
  * call of this library that allocates and synchronises: it runs a 64-block
  * probe on the default stream and waits for it - a set-up call, not one for a
  * serving loop or a stream under capture (mint_xcd_map is the asynchronous
- * form). */
+ * form).  `xcds` is the number of distinct XCDs the probe's blocks landed on;
+ * when that is 8 but some aligned group of 8 consecutive blocks did not land
+ * on 8 different XCDs - the dealing MINT_PLACE_LOCAL is built on - it is
+ * reported as 0 and MINT_PLACE_SPREAD is the placement to use.  (A launch
+ * with MINT_PLACE_LOCAL on a device that deals otherwise loses no data
+ * silently: some (channel, position) is then served twice and another not at
+ * all, the neighbours' bounded waits run out, status word 0 says 1 and
+ * in-place buffers are left partly updated.) */
 int mint_device_info(int* compute_units, int* xcds, int* wave_size);
 
 /* XCC_ID of the XCD each of `blocks` thread blocks of a 1-D launch lands on

@@ -474,7 +474,10 @@ class VirtualComm:
                 _lib.check(self._lib.mint_ring_launch(d, stream), "mint_ring_launch")
 
     def check(self) -> None:
-        """Synchronise and raise ``RingTimeout`` if a wait gave up."""
+        """Synchronise and raise ``RingTimeout`` if a wait gave up.  Only the
+        first failure is recorded; every launch queued behind it found the
+        abort word set and gave up at its first wait, so the outputs of all
+        launches since the last clean check are unspecified."""
         torch.cuda.synchronize(self.device)
         st = self.status.cpu().tolist()
         if st[0] != 0:
@@ -486,7 +489,8 @@ class VirtualComm:
                     "use placement spread (and cache_policy 0) on this device")
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
-                f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]}")
+                f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]} "
+                "(outputs of every launch since the last check are unspecified)")
 
 
 _default_comm: VirtualComm | None = None

@@ -373,6 +373,17 @@ int mint_device_info(int* compute_units, int* xcds, int* wave_size) {
         uint32_t mask = 0;
         for (uint32_t v : h) mask |= 1u << (v & 31u);
         *xcds = __builtin_popcount(mask);
+        // MINT_PLACE_LOCAL relies on more than the count: every aligned group
+        // of 8 consecutive blocks has to land on 8 different XCDs.  Where the
+        // probe does not show that, the device is reported as not dealing
+        // regularly (0) and callers stay with MINT_PLACE_SPREAD.
+        if (*xcds == kXcds) {
+            for (int g = 0; g < 64; g += kXcds) {
+                uint32_t seen = 0;
+                for (int i = 0; i < kXcds; ++i) seen |= 1u << (h[g + i] & 31u);
+                if (__builtin_popcount(seen) != kXcds) *xcds = 0;
+            }
+        }
     }
     return MINT_OK;
 }

@@ -21,7 +21,8 @@ def dev_bytes(a: np.ndarray, dev) -> torch.Tensor:
 def test_device_is_mi355x_shaped(lib):
     cu, xcd, wave = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     assert lib.mint_device_info(cu, xcd, wave) == 0
-    assert wave.value == 64 and cu.value > 0 and xcd.value >= 1
+    # 8 XCDs, and the probe found every aligned group of 8 blocks on 8 different ones
+    assert wave.value == 64 and cu.value > 0 and xcd.value == 8
 
 
 def test_blocks_are_dealt_round_robin_over_xcds(lib, dev):
