@@ -244,6 +244,25 @@ def config5(reps: int, max_log2: int) -> None:
                      shard_bytes=shard, us=round(ms * 1e3, 2),
                      alg_gbps=round((3 * world - 2) * S / ms / 1e6, 1), hbm_bytes=world * S,
                      busbw_gbps=round(shard * (world - 1) / ms / 1e6, 1), ok=ok)
+                if label == "tuned" and proto == 0 and log2 in (16, 20, 23, 27):
+                    # the temporal schedule (6_allgather.py:25-77): row after row
+                    # through one pipeline; same bytes
+                    for b in bufs:
+                        b.zero_()
+                    for r in range(world):
+                        bufs[r][r] = want[r]
+                    td = comm.make_op(_lib.OP_ALLGATHER_TEMPORAL, _lib.BYTES, shard, ptrs, ptrs,
+                                      list(range(world)) + [0], row_stride=shard,
+                                      protocol=_lib.PROTO_LL128)
+                    comm.launch(td)
+                    comm.check()
+                    tok = all(torch.equal(b.view(torch.int16), want.view(torch.int16)) for b in bufs)
+                    tms = time_ms(lambda: comm.launch(td), (reps if log2 < 24 else max(2, reps // 2)) * 4)
+                    comm.check()
+                    emit(config=5, op="allgather", protocol=name, staging="tuned, temporal",
+                         world=world, shard_bytes=shard, us=round(tms * 1e3, 2),
+                         alg_gbps=round((3 * world - 2) * S / tms / 1e6, 1), hbm_bytes=world * S,
+                         busbw_gbps=round(shard * (world - 1) / tms / 1e6, 1), ok=tok)
                 if label == "tuned" and log2 <= 16 and log2 % 2 == 1:
                     # the same launch as 20 nodes of a HIP graph (epoch in device
                     # memory, advanced by a small kernel in front of every launch):

@@ -65,7 +65,7 @@ typedef enum {
                                   destination's staging (input[] and output[] must
                                   not overlap) */
     MINT_OP_TREE_BROADCAST = 7, /* broadcast and reduce over a binary tree, an open */
-    MINT_OP_TREE_REDUCE = 8     /* item of the reference's roadmap (README.md:52-55).
+    MINT_OP_TREE_REDUCE = 8,    /* item of the reference's roadmap (README.md:52-55).
                                   The tree is laid over ring[] turned so that the
                                   root comes first: node h (0 = root) has parent
                                   (h - 1) / 2 and children 2h + 1, 2h + 2.  Buffers
@@ -74,6 +74,12 @@ typedef enum {
                                   rounding per addition.  LL128 only.  slot_bytes
                                   of a TREE_REDUCE holds two shares (one per
                                   child). */
+    MINT_OP_ALLGATHER_TEMPORAL = 9 /* 6_allgather.py:25-77, the schedule the
+                                  reference's allgather launches (:157): the whole
+                                  grid moves rank 0's row round the ring, then rank
+                                  1's, ...; one pipeline, so slot_bytes holds one
+                                  row's share.  Same descriptor and same result as
+                                  MINT_OP_ALLGATHER.  LL128 only. */
 } mint_op;
 typedef enum {
     MINT_PLACE_SPREAD = 0,  /* ring neighbours on consecutive blocks (adjacent XCDs) */
@@ -133,7 +139,7 @@ typedef struct {
                               words sit behind the slots, outside a buffer
                               that only holds nslots * slot_bytes) */
     uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE/TREE_*: bytes of the
-                              buffer; ALLGATHER/REDUCESCATTER/ALLTOALL: bytes of
+                              buffer; ALLGATHER(_TEMPORAL)/REDUCESCATTER/ALLTOALL: bytes of
                               one row */
     uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER/ALLTOALL: bytes between rows */
     uint32_t slot_bytes;   /* staging bytes of one step over all pipelines;
@@ -264,8 +270,8 @@ int mint_ring_grid_blocks(const mint_ring_op* op);
  * 1024 for Simple), recv_offset[i] / send_offset[i] (byte offset of the
  * block's 1 KiB message inside the staging of the rank it is received in /
  * sent to).  Any output array may be NULL; at most max_entries are written,
- * *n_entries is the full count.  Needs no GPU.  The tree ops are not listed
- * (MINT_ERR_ARG). */
+ * *n_entries is the full count.  Needs no GPU.  The tree ops and the temporal
+ * allgather are not listed (MINT_ERR_ARG). */
 int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
                        uint32_t max_entries, uint32_t* step, uint32_t* block,
                        uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries);

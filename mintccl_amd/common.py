@@ -175,7 +175,8 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
     if op == _lib.OP_ALLREDUCE:
         pipes *= 2                # a slot is shared by (pipeline, phase): two phases
     npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_BROADCAST: world,
-            _lib.OP_ALLGATHER: world, _lib.OP_ALLREDUCE: 2 * world - 1}.get(op, world + 1)
+            _lib.OP_ALLGATHER: world, _lib.OP_ALLGATHER_TEMPORAL: world,
+            _lib.OP_ALLREDUCE: 2 * world - 1}.get(op, world + 1)
     receivers = max(1, min(npos - 1, world))
     if op == _lib.OP_ALLREDUCE:
         npos = (npos + 1) // 2    # `pipes` already counts both phases

@@ -7,6 +7,7 @@
 
 #include "kernels.hpp"
 #include "ring_launch.hpp"
+#include "temporal.hpp"
 #include "tree.hpp"
 
 using namespace mint;
@@ -37,7 +38,8 @@ bool reducing(int op) {
            op == MINT_OP_TREE_REDUCE;
 }
 bool over_tree(int op) { return op == MINT_OP_TREE_BROADCAST || op == MINT_OP_TREE_REDUCE; }
-static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE == OP_TREE_REDUCE,
+static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE == OP_TREE_REDUCE &&
+                  MINT_OP_ALLGATHER_TEMPORAL == OP_ALLGATHER_TEMPORAL,
               "op codes");
 
 // Everything the launch derives from the descriptor.  `for_launch`: also
@@ -46,11 +48,12 @@ static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE
 int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
               const mint_ring_debug* dbg = nullptr) {
     if (!op || !plan) return MINT_ERR_ARG;
-    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_TREE_REDUCE) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLGATHER_TEMPORAL) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
-    // the tree kernels speak LL128 only
-    if (over_tree(op->op) && op->protocol != MINT_PROTO_LL128) return MINT_ERR_ARG;
+    // the tree kernels and the temporal allgather speak LL128 only
+    const bool temporal = op->op == MINT_OP_ALLGATHER_TEMPORAL;
+    if ((over_tree(op->op) || temporal) && op->protocol != MINT_PROTO_LL128) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
     if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
     if (op->cache_policy < 0 || op->cache_policy > 2) return MINT_ERR_ARG;
@@ -76,8 +79,10 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     const bool allreduce = op->op == MINT_OP_ALLREDUCE;
     const bool alltoall = op->op == MINT_OP_ALLTOALL;
     const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER ||
-                         allreduce || alltoall;
-    a.pipes = alltoall ? op->world * op->world : (rowwise ? op->world : 1);
+                         allreduce || alltoall || temporal;
+    // (the temporal allgather moves its `world` rows one after the other
+    // through one pipeline)
+    a.pipes = alltoall ? op->world * op->world : (rowwise && !temporal ? op->world : 1);
     a.phases = allreduce ? 2 : 1;
     // a rank receives from every pipeline that passes through it: one share of
     // its slots per pipeline and phase; in an alltoall, one per source rank
@@ -120,9 +125,9 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         }
         case MINT_OP_ALLTOALL: a.hops = 1; break;
         default:
-            a.hops = op->op == MINT_OP_ALLGATHER ? op->world - 1
-                     : allreduce                 ? 2 * op->world - 2
-                                                 : op->world;
+            a.hops = op->op == MINT_OP_ALLGATHER || temporal ? op->world - 1
+                     : allreduce                             ? 2 * op->world - 2
+                                                             : op->world;
             for (int p = 0; p < op->world; ++p) a.start[p] = (uint8_t)index_of(p);
     }
 
@@ -161,7 +166,13 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         if (receives && (!op->staging[rank] || !aligned16(op->staging[rank])))
             return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
     }
-    for (int p = 0; p < a.pipes && !plan->empty && !over_tree(op->op); ++p) {
+    for (int r = 0; r < op->world && temporal && !plan->empty; ++r) {
+        // every rank is origin once and receiver world - 1 times
+        if (!op->input[r] || !op->output[r]) return MINT_ERR_ARG;
+        if (!op->staging[r] || !aligned16(op->staging[r]))
+            return op->staging[r] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
+    }
+    for (int p = 0; p < a.pipes && !plan->empty && !over_tree(op->op) && !temporal; ++p) {
         for (int h = 0; h <= a.hops; ++h) {
             const int rank = alltoall ? (h == 0 ? p / op->world : p % op->world)
                                       : a.cyc[(a.start[p] + h) % a.cyc_len];
@@ -210,6 +221,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     a.nblocks = (uint32_t)nblocks;
     a.steps = (a.nblocks + a.step_blocks - 1) / a.step_blocks;
     if (a.steps > kMaxSteps) return MINT_ERR_TOO_LARGE;
+    // (the temporal allgather numbers its steps through all rows)
+    if (temporal && (uint64_t)a.steps * (uint64_t)op->world > kMaxSteps) return MINT_ERR_TOO_LARGE;
     a.credit_off = a.nslots * a.slot_bytes;
     if (op->credit_offset) {
         if (op->credit_offset < a.credit_off || op->credit_offset % 256) return MINT_ERR_GEOMETRY;
@@ -577,7 +590,8 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
     const int err = make_plan(op, &plan);
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
-    if (over_tree(op->op)) return MINT_ERR_ARG;     // listed for the ring walks only
+    if (over_tree(op->op) || op->op == MINT_OP_ALLGATHER_TEMPORAL)
+        return MINT_ERR_ARG;                        // listed for the ring walks only
     const RingArgs& a = plan.args;
     if (pipeline < 0 || pipeline >= a.pipes || position < 0 || position > a.hops || wave < 0 ||
         wave >= a.waves)

@@ -3,6 +3,7 @@
 #include <atomic>
 
 #include "ring_launch.hpp"
+#include "temporal.hpp"
 #include "tree.hpp"
 
 #ifndef MINT_FAMILY_DT
@@ -130,8 +131,41 @@ int launch_tree(const Plan& plan, hipStream_t stream) {
     return launch_status();
 }
 
+// Allgather, temporal schedule (LL128, bytes): one wavefront per (rank,
+// wave-channel).
+template <int CP>
+int launch_temporal(const Plan& plan, hipStream_t stream) {
+    void (*kernel)(const RingArgs) = temporal_kernel<CP>;
+    static std::atomic<int> cached[9] = {};          // [threads / 64]
+    static std::atomic<int> cus{0};
+    std::atomic<int>& memo = cached[plan.threads / 64];
+    int per_cu = memo.load(std::memory_order_relaxed);
+    if (per_cu == 0) {
+        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
+        if (per_cu < 0) return MINT_ERR_HIP;
+        memo.store(per_cu, std::memory_order_relaxed);
+    }
+    int ncu = cus.load(std::memory_order_relaxed);
+    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
+    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
+                       plan.args);
+    return launch_status();
+}
+
 template <int DT>
 int launch_family(const Plan& plan, int protocol, int cache_policy, hipStream_t stream) {
+    if (plan.args.op == OP_ALLGATHER_TEMPORAL) {
+        if constexpr (DT == DT_BYTES) {
+            switch (cache_policy) {
+                case 0: return launch_temporal<0>(plan, stream);
+                case 1: return launch_temporal<1>(plan, stream);
+                default: return launch_temporal<2>(plan, stream);
+            }
+        } else {
+            return MINT_ERR_ARG;
+        }
+    }
     if (plan.args.op == OP_TREE_BROADCAST || plan.args.op == OP_TREE_REDUCE) {
         switch (cache_policy) {
             case 0: return launch_tree<DT, 0>(plan, stream);

@@ -131,7 +131,9 @@ def test_plan_geometry_without_a_gpu():
 
 @pytest.mark.parametrize("kw,err", [
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
-    (dict(op=9), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=10), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES, protocol=_lib.PROTO_SIMPLE,
+          waves_per_channel_group=128), _lib.ERR_ARG),   # LL128 only
     (dict(op=_lib.OP_TREE_REDUCE, protocol=_lib.PROTO_SIMPLE, waves_per_channel_group=128),
      _lib.ERR_ARG),                                      # the tree kernels speak LL128 only
     (dict(op=_lib.OP_TREE_REDUCE, dtype=_lib.BYTES, waves_per_channel_group=128), _lib.ERR_ARG),
@@ -220,6 +222,29 @@ def test_tree_plans_without_a_gpu():
     n = ctypes.c_uint32(0)
     d = make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=128)
     assert L.mint_ring_schedule(d, 0, 0, 0, 0, None, None, None, None, ctypes.byref(n)) == _lib.ERR_ARG
+
+
+def test_temporal_allgather_plan_without_a_gpu():
+    """6_allgather.py:25-77: one pipeline of `world` positions that moves the rows
+    one after the other; a slot holds one row's share."""
+    L = _lib.lib()
+    d = make_op(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES, waves_per_channel_group=128)
+    assert L.mint_ring_grid_blocks(d) == 8 * 32
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256
+    # the same slot takes 8 x 64 blocks of the spatial schedule or 512 of this one
+    assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES,
+                                           waves_per_channel_group=512)) == 8 * 128
+    assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES,
+                                           waves_per_channel_group=512)) == _lib.ERR_GEOMETRY
+    d.staging[5] = 0
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
+    # steps are numbered through all rows: 8 x 2^17 of them do not fit the 20-bit tag field
+    d = make_op(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES, waves_per_channel_group=1,
+                slot_bytes=1024, count_bytes=960 << 17, row_stride=960 << 17)
+    assert L.mint_ring_grid_blocks(d) == _lib.ERR_TOO_LARGE
+    d = make_op(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES, waves_per_channel_group=1,
+                slot_bytes=8192, count_bytes=960 << 17, row_stride=960 << 17)
+    assert L.mint_ring_grid_blocks(d) > 0
 
 
 def test_launch_refuses_undersized_staging_before_touching_the_gpu():

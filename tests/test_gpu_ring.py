@@ -256,6 +256,82 @@ def test_allgather(dev, world, n, proto):
     assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
 
 
+def run_allgather_temporal(comm, bufs):
+    from mintccl_amd.allgather import allgather
+    comm.run(lambda r: allgather(bufs[r], comm, schedule="temporal"))
+    comm.check()
+
+
+@pytest.mark.parametrize("world", WORLDS)
+@pytest.mark.parametrize("n", [8, 480, 488, 65536])
+def test_allgather_temporal_schedule(dev, world, n):
+    """6_allgather.py:25-77: the rows go round one after the other; same bytes
+    as the spatial schedule."""
+    host = [uniform(world * n, -1.0, 1.0, 40 + r).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world)
+    run_allgather_temporal(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+
+
+@pytest.mark.parametrize("world", [3, 8])
+@pytest.mark.parametrize("geometry", [dict(buff_size_=2 * 16 * 1024, nslots=2, waves_per_rank=16),
+                                      dict(buff_size_=3 * 64 * 1024, nslots=3, waves_per_rank=32),
+                                      dict(buff_size_=5 * 8 * 1024, nslots=5, waves_per_rank=8,
+                                           placement=0, cache_policy=0),
+                                      dict(buff_size_=2 * 64 * 1024, nslots=2, waves_per_rank=64,
+                                           placement=1, cache_policy=2)])
+def test_allgather_temporal_many_steps_through_few_slots(dev, world, geometry):
+    # 100003 halves per row: 209 blocks, so every row takes several steps and
+    # the step count carries on from row to row through the same slots; the
+    # link into a row's owner is idle while that row goes round
+    n = 100003
+    host = [uniform(world * n, -1.0, 1.0, 50 + r).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    comm = make_comm(world, **geometry)
+    run_allgather_temporal(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    # and again on the same staging, then the spatial schedule on top of it
+    bufs = [h.to(dev) for h in host]
+    run_allgather_temporal(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    bufs = [h.to(dev) for h in host]
+    run_allgather(comm, bufs)
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+
+
+def test_allgather_temporal_over_a_permuted_ring_and_by_env(dev, monkeypatch):
+    from mintccl_amd import topology
+    from mintccl_amd.allgather import allgather
+    world, n = 5, 30001
+    comm = make_comm(world)
+    comm.topology = topology.uniform_topology(world)
+    comm._ring_cache = (comm.topology, [0, 2, 4, 1, 3, 0])
+    host = [uniform(world * n, -1.0, 1.0, 60 + r).reshape(world, n) for r in range(world)]
+    bufs = [h.to(dev) for h in host]
+    monkeypatch.setenv("MINTCCL_ALLGATHER", "temporal")
+    comm.run(lambda r: allgather(bufs[r], comm))
+    comm.check()
+    assert same(bufs, ring.allgather([as_bytes(h) for h in host]))
+    # one pipeline: 63 blocks per row -> 64 wave-channels per rank, 16 thread blocks each
+    assert comm.last_grid == world * 16
+
+
+def test_allgather_temporal_8_x_8mib(dev):
+    world, n = 8, 4 << 20
+    g = torch.Generator(device=dev).manual_seed(5)
+    bufs = []
+    for r in range(world):
+        b = torch.zeros(world, n, dtype=torch.float16, device=dev)
+        b[r].uniform_(-1, 1, generator=g)
+        bufs.append(b)
+    want = torch.stack([bufs[r][r] for r in range(world)])
+    comm = make_comm(world)
+    run_allgather_temporal(comm, bufs)
+    for b in bufs:
+        assert torch.equal(b, want)
+
+
 @pytest.mark.parametrize("world", [2, 4, 8])
 def test_xcd_local_policy_all_collectives(dev, world):
     # stores that stay in one XCD's L2: every collective, ragged sizes, many
