@@ -228,6 +228,8 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
  *   4  a 16-byte-per-lane store of the f16 sum of the two into the other slot,
  *   8  (with 1) the own block is loaded straight into LDS (buffer_load ... lds)
  *      and read from there, instead of into registers,
+ *  16  (without 1 and 8) a streaming store of the block back into `rows`, as a
+ *      copying position saves what it received (`rows` is written),
  * with no flags and nobody waiting for anybody.  The launch takes what the
  * device needs for that mix of accesses however well a ring schedules them:
  * the yardstick beside mint_copy_simple and mint_read_xor.  `sink` (device

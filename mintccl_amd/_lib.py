@@ -39,6 +39,9 @@ HIPCC_FLAGS = [
     # packed FP32 instructions are kept out of all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
+    # the compiler reports every kernel's registers and scratch memory; build()
+    # refuses a kernel that uses scratch (see there)
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 
@@ -104,6 +107,21 @@ SYMBOLS = {
 _lib = None
 
 
+def kernels_with_scratch(remarks: str) -> list[str]:
+    """Names of the kernels whose ``-Rpass-analysis=kernel-resource-usage``
+    remarks report a non-zero scratch size."""
+    import re
+    out, name = [], "?"
+    for line in remarks.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and int(m.group(1)) > 0:
+            out.append(f"{name} ({m.group(1)} bytes per lane)")
+    return out
+
+
 def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | None = None) -> str:
     """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree).
 
@@ -127,13 +145,19 @@ def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | N
             print(" ".join(cmd))
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
                                             text=True)))
-    errors = []
+    errors, spilling = [], []
     for cmd, proc in procs:
         _, err = proc.communicate()
         if proc.returncode != 0:
             errors.append(f"{' '.join(cmd)}\n{err}")
+        spilling += kernels_with_scratch(err)
     if errors:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
+    if spilling:
+        # A walk whose locals the optimiser could not keep in registers (it
+        # happens when closures capture closures) still computes the right
+        # bytes, five times slower: fail the build instead.
+        raise RuntimeError("kernels that use scratch memory: " + ", ".join(spilling))
     link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out,
             *[obj for _, _, obj in units]]
     if verbose:

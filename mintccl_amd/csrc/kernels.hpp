@@ -144,10 +144,15 @@ __global__ void __launch_bounds__(256) step_mix_kernel(const uint8_t* __restrict
             own = ll_fetch_raw(rows, 0, i * waves + wave, true, m);
         }
         const u32x4 x = add_rn<DT_F16>(own, got);
+        // WHAT & 16: the block also goes back to HBM, as a copying position
+        // saves what it received (a streaming store of the 960 raw bytes)
+        if (WHAT & 16)
+            ll_save_raw(const_cast<uint8_t*>(rows), (uint64_t)waves * iters * kBlockRawLL,
+                        i * waves + wave, true, m, x);
         if (WHAT & 4) st128<CP_NONE>(win, slot0 + ((i + 1u) & 1u) * kBlockMsg + m.lane * 16u, x);
-        else acc ^= x;
+        else if (!(WHAT & 16)) acc ^= x;
     }
-    if (!(WHAT & 4) && acc.x == 0x9E3779B9u && acc.y == 0x85EBCA6Bu && acc.z == 0xC2B2AE35u)
+    if (!(WHAT & 20) && acc.x == 0x9E3779B9u && acc.y == 0x85EBCA6Bu && acc.z == 0xC2B2AE35u)
         sink[0] = acc.w;     // keeps the loads alive; practically never taken
 }
 

@@ -449,14 +449,14 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
 
 int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
                   int waves, int iters, int what, void* sink, void* stream) {
-    if (waves <= 0 || iters <= 0 || what < 1 || what > 15 || (what & 9) == 8) return MINT_ERR_ARG;
-    if ((what & 1) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
+    if (waves <= 0 || iters <= 0 || what < 1 || what > 31 || (what & 9) == 8) return MINT_ERR_ARG;
+    if ((what & 17) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
         return MINT_ERR_ARG;
     if ((size_t)waves * (size_t)iters >= (1ull << 32)) return MINT_ERR_TOO_LARGE;
     if ((what & 6) && (!staging || staging_bytes < (size_t)waves * 2u * kBlockMsg)) return MINT_ERR_ARG;
     if ((what & 6) && staging_bytes >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
     if ((what & 6) && !aligned16(staging)) return MINT_ERR_ALIGN;
-    if (!(what & 4) && !sink) return MINT_ERR_ARG;
+    if (!(what & 20) && !sink) return MINT_ERR_ARG;
     void (*kernel)(const uint8_t*, uint8_t*, uint32_t, uint32_t, uint32_t, uint32_t*) = nullptr;
     switch (what) {
         case 1: kernel = step_mix_kernel<1>; break;
@@ -469,7 +469,12 @@ int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t sta
         case 9: kernel = step_mix_kernel<9>; break;
         case 11: kernel = step_mix_kernel<11>; break;
         case 13: kernel = step_mix_kernel<13>; break;
-        default: kernel = step_mix_kernel<15>; break;
+        case 15: kernel = step_mix_kernel<15>; break;
+        case 16: kernel = step_mix_kernel<16>; break;
+        case 18: kernel = step_mix_kernel<18>; break;
+        case 20: kernel = step_mix_kernel<20>; break;
+        case 22: kernel = step_mix_kernel<22>; break;
+        default: return MINT_ERR_ARG;
     }
     const unsigned blocks = ((unsigned)waves + 3u) / 4u;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, as_stream(stream),

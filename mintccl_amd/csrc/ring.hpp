@@ -309,6 +309,13 @@ __device__ __forceinline__ LdsPort lds_port(MINT_LDS uint8_t* base, int j, uint3
     return port;
 }
 
+// The lambdas of the walk are inlined early and kept shallow: every level of
+// lambdas capturing lambdas by reference takes the optimiser one more round
+// to dissolve, and what it does not dissolve stays in scratch memory (a third
+// level left 2.8 KB per lane there and made the copying collectives five
+// times slower; the build refuses kernels that use scratch).
+#define MINT_INLINE_LAMBDA __attribute__((always_inline))
+
 // The walk of one wave-channel along its rows, specialised by what its
 // position does (the flags are compile-time constants so that the loop of an
 // origin, an adder, a copier or a sink carries no tests for the other roles).
@@ -362,7 +369,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     using Group = mint::Group<U>;
     // load_ll128 of the wave's own rows for one group: only the loads;
     // ll_arrange finishes the job where the values are needed.
-    auto load_own = [&](const Group& q, u32x4 (&v)[U]) {
+    auto load_own = [&](const Group& q, u32x4 (&v)[U]) MINT_INLINE_LAMBDA {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             v[u] = u32x4{0u, 0u, 0u, 0u};
@@ -381,7 +388,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // loads are issued unconditionally and always land inside the row (what
     // they bring is only used if the group turns out to be a whole one).
     // Needs nfull >= 1.
-    auto fetch_ahead = [&](const Group& q, u32x4 (&v)[U]) {
+    auto fetch_ahead = [&](const Group& q, u32x4 (&v)[U]) MINT_INLINE_LAMBDA {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t g = q.g[u] < nfull ? q.g[u] : nfull - 1u;
@@ -397,7 +404,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // wavefront's operations in order, so the fetcher that sees the new
     // `consumed` knows the reads before it have been done.
     uint32_t lds_taken = 0, lds_entry = 0;
-    auto lds_take = [&](u32x4 (&x)[U]) -> bool {
+    auto lds_take = [&](u32x4 (&x)[U]) MINT_INLINE_LAMBDA -> bool {
         for (uint32_t spins = 0; lds_count(port.produced) <= lds_taken; ++spins) {
             if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) return false;
             __builtin_amdgcn_s_sleep(1);
@@ -444,7 +451,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // flight: it has a whole group's time to come back from HBM.  The other
     // groups (the ragged end of a row, a step that is only partly filled) take
     // the guarded body and load their own rows on the spot.
-    auto run_group = [&](auto whole_tag, auto parity_tag) -> bool {
+    auto run_group = [&](auto whole_tag, auto parity_tag) MINT_INLINE_LAMBDA -> bool {
         constexpr bool WHOLE = decltype(whole_tag)::value;
         constexpr int P = decltype(parity_tag)::value;
         u32x4 (&v)[U] = rows[P];
@@ -619,14 +626,14 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             u32x4 rr[2][U], vv[2][U];
             uint64_t cw[2] = {0, 0};
             uint32_t step = 0, slot = 0;
-            auto poll_step = [&](uint32_t at_slot, u32x4 (&r)[U]) {
+            auto poll_step = [&](uint32_t at_slot, u32x4 (&r)[U]) MINT_INLINE_LAMBDA {
                 const uint32_t base = at_slot * a.slot_bytes + share_recv * a.step_msg;
 #pragma unroll
                 for (int u = 0; u < U; ++u)
                     r[u] = ld128<LDCP>(own, base + ((uint32_t)u * W + (uint32_t)w) * kBlockMsg +
                                                 m.lane * 16u);
             };
-            auto fetch_step = [&](uint32_t of_step, u32x4 (&x)[U]) {
+            auto fetch_step = [&](uint32_t of_step, u32x4 (&x)[U]) MINT_INLINE_LAMBDA {
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     uint32_t g = of_step * a.step_blocks + (uint32_t)u * W + (uint32_t)w;
@@ -635,11 +642,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 }
             };
             uint64_t* const pad = own_tail + 8;
-            auto store_pad = [&]() {
+            auto store_pad = [&]() MINT_INLINE_LAMBDA {
                 if (STCP == CP_NONE) st64_local(pad, 0ull);
                 else st64_agent(pad, 0ull);
             };
-            auto give_up = [&]() {
+            auto give_up = [&]() MINT_INLINE_LAMBDA {
                 report_timeout(a.status, p, h, w, step);
                 __builtin_amdgcn_endpgm();
             };
@@ -656,7 +663,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             if (role.recv) store_pad();
             compiler_fence();
             if (role.load) fetch_step(1, vv[1]);
-            auto whole_step = [&](auto phase) {
+            auto whole_step = [&](auto phase) MINT_INLINE_LAMBDA {
                 constexpr int B = decltype(phase)::value, B1 = B ^ 1;
                 const uint32_t next_slot = slot + 1 == a.nslots ? 0 : slot + 1;
                 const uint32_t tag = (epoch << 20) | (step + 1u);

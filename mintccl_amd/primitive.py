@@ -48,10 +48,11 @@ def step_mix(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int
     """The memory accesses of ``waves`` x ``iters`` ring steps with no ring around
     them (``what``: 1 own-row loads from ``rows``, 2 loads from ``staging``,
     4 stores into ``staging``, 8 with 1: own rows loaded straight into LDS
-    instead of into registers): the yardstick for what the device can do with
+    instead of into registers, 16 without 1: the block is stored back into
+    ``rows``): the yardstick for what the device can do with
     the ring kernels' mix of accesses."""
     ref = rows if rows is not None else staging
-    if sink is None and not what & 4:
+    if sink is None and not what & 20:
         sink = torch.zeros(1, dtype=torch.int32, device=ref.device)
     nb = lambda t: 0 if t is None else t.numel() * t.element_size()
     ptr = lambda t: None if t is None else t.data_ptr()

@@ -3,7 +3,8 @@ waits for anything: ``python -m mintccl_amd.yardsticks`` prints, one JSON line
 each, the copy and read bandwidth of the library's own kernels on 1 GiB and
 the time of ``mint_step_mix`` - per wavefront and step a 960-byte own-row load
 from HBM, a 1 KiB load from and a 1 KiB store into a private staging slot, in
-every combination, also with the own rows loaded straight into LDS - for the block count of the headline launch (8 ranks x
+every combination, also with the own rows loaded straight into LDS, and the
+mix of a copying position (staging load, staging store, store to HBM) - for the block count of the headline launch (8 ranks x
 256 MiB: 2,517,120 blocks of 1 KiB) spread over different numbers of
 wavefronts.  The ring kernels do exactly these accesses plus their flags, so
 these times are what they are measured against.  No counterpart in the
@@ -52,7 +53,10 @@ def main(argv: list[str]) -> int:
     what = (("own rows", 1), ("staging load", 2), ("staging store", 4), ("staging load + store", 6),
             ("own rows + staging store", 5), ("own rows + staging load", 3), ("all three", 7),
             ("own rows into LDS", 9), ("own rows into LDS + staging store", 13),
-            ("all three, own rows into LDS", 15))
+            ("all three, own rows into LDS", 15),
+            # what a copying position does: staging load, save to HBM, staging store
+            ("HBM store", 16), ("staging load + HBM store", 18), ("staging store + HBM store", 20),
+            ("staging load + staging store + HBM store", 22))
     for waves in waves_list:
         iters = -(-BLOCKS // waves)
         staging = torch.zeros(waves * 2048, dtype=torch.uint8, device=dev)

@@ -201,3 +201,32 @@ def test_step_mix_moves_what_it_says(dev, via_lds):
     assert torch.equal(staging, before)
     primitive.step_mix(rows, staging, waves, iters, what=7 | via_lds)
     torch.cuda.synchronize()
+
+
+def test_step_mix_saves_what_it_loads_from_staging(dev):
+    """Bit 16: the block a wave took out of its staging slot goes back to HBM in
+    the raw layout (lane l, l % 4 != 3: 16 bytes at vector l - l // 4; a flag
+    lane: its 12 payload bytes behind the 48 vectors)."""
+    from mintccl_amd import primitive
+    waves, iters = 21, 4
+    rows = torch.zeros(waves * iters * 960, dtype=torch.uint8, device=dev)
+    staging = (torch.rand(waves * 1024, device=dev) + 1).to(torch.float16).view(torch.uint8)
+    before = staging.clone()
+    primitive.step_mix(rows, staging, waves, iters, what=2 | 16)
+    torch.cuda.synchronize()
+    assert torch.equal(staging, before)
+    r, s = rows.cpu().numpy(), staging.cpu().numpy()
+    for w in (0, 5, waves - 1):
+        for i in (0, iters - 1):
+            block = r[(i * waves + w) * 960:][:960]
+            slot = s[w * 2048 + (i & 1) * 1024:][:1024]
+            for lane in range(64):
+                if lane % 4 != 3:
+                    vec = lane - lane // 4
+                    assert (block[vec * 16: vec * 16 + 16] == slot[lane * 16: lane * 16 + 16]).all()
+                else:
+                    at = 768 + 12 * (lane // 4)
+                    assert (block[at: at + 12] == slot[lane * 16: lane * 16 + 12]).all()
+    primitive.step_mix(rows, staging, waves, iters, what=2 | 4 | 16)       # only has to run
+    torch.cuda.synchronize()
+
