@@ -115,6 +115,35 @@ def test_static_launch_ll128_after_simple_and_other_geometries(dev, lib):
             assert np.array_equal(as_bytes(g[r]), want[r]), (n, r)
 
 
+@pytest.mark.gpu
+def test_static_launch_of_the_tree_and_the_temporal_schedule(dev, lib):
+    """The newer walks through the same static array: a reduce up the binary tree
+    (two shares per slot) and the allgather that moves row after row."""
+    status = torch.zeros(4, dtype=torch.int64, device=dev)
+    n = 30011
+    host = [uniform(n, -1.0, 1.0, 70 + r) for r in range(WORLD)]
+    bufs = [h.to(dev) for h in host]
+    d = descriptor(_lib.OP_TREE_REDUCE, _lib.F16, _lib.PROTO_LL128, n * 2,
+                   [t.data_ptr() for t in bufs], status, root=5, slot_bytes=2 * 32 * 1024, nslots=3,
+                   waves=32)
+    launch_static(lib, d)
+    assert ok(status)
+    want = ring.tree_reduce([as_bytes(h) for h in host], 5, "f16")
+    for r in range(WORLD):
+        assert np.array_equal(as_bytes(bufs[r]), want[r]), r
+    m = 9001
+    host = [uniform(WORLD * m, -1.0, 1.0, 80 + r).reshape(WORLD, m) for r in range(WORLD)]
+    g = [h.to(dev) for h in host]
+    d = descriptor(_lib.OP_ALLGATHER_TEMPORAL, _lib.BYTES, _lib.PROTO_LL128, m * 2,
+                   [t.data_ptr() for t in g], status, slot_bytes=8 * 1024, nslots=2, waves=8)
+    d.row_stride = m * 2
+    launch_static(lib, d)
+    assert ok(status)
+    want = ring.allgather([as_bytes(h) for h in host])
+    for r in range(WORLD):
+        assert np.array_equal(as_bytes(g[r]), want[r]), r
+
+
 def test_static_launch_refuses_what_does_not_fit_the_array():
     """Size limits are checked before any device is touched."""
     L = _lib.lib()
