@@ -265,6 +265,23 @@ def test_launch_refuses_undersized_staging_before_touching_the_gpu():
     assert L.mint_ring_launch_debug(d, dbg, None) == _lib.ERR_ARG
 
 
+def test_build_refuses_kernels_that_use_scratch():
+    """The build reads hipcc's kernel-resource-usage remarks: a kernel whose
+    locals were left in scratch memory computes the right bytes several times
+    slower, so it is reported by name."""
+    remarks = """\
+a.hpp:9:1: remark: Function Name: _ZN4mint11ring_kernelILi0ELi3ELi2ELi1EEEvNS_8RingArgsE [-Rpass-analysis=kernel-resource-usage]
+a.hpp:9:1: remark:     VGPRs: 91 [-Rpass-analysis=kernel-resource-usage]
+a.hpp:9:1: remark:     ScratchSize [bytes/lane]: 2832 [-Rpass-analysis=kernel-resource-usage]
+a.hpp:9:1: remark: Function Name: _ZN4mint11tree_kernelILi0ELi2EEEvNS_8RingArgsE [-Rpass-analysis=kernel-resource-usage]
+a.hpp:9:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+"""
+    bad = _lib.kernels_with_scratch(remarks)
+    assert bad == ["_ZN4mint11ring_kernelILi0ELi3ELi2ELi1EEEvNS_8RingArgsE (2832 bytes per lane)"]
+    assert _lib.kernels_with_scratch("") == []
+    assert "-Rpass-analysis=kernel-resource-usage" in _lib.HIPCC_FLAGS
+
+
 def test_missing_library_fails_loudly(tmp_path):
     code = ("import mintccl_amd._lib as l; l.SO_PATH=%r; l._lib=None\n"
             "try:\n    l.lib()\nexcept RuntimeError as e:\n    print('RAISED', 'no CPU fallback' in str(e))\n"
