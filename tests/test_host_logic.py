@@ -30,16 +30,20 @@ def test_largest_divisor(n, cap, want):
 
 
 @pytest.mark.parametrize("world", [2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("row_blocks", [None, 1, 37, 5000])
 @pytest.mark.parametrize("op", [_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_REDUCE, _lib.OP_ALLGATHER,
-                                _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL])
-def test_tuned_geometry_is_always_launchable(op, world):
+                                _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_ALLTOALL,
+                                _lib.OP_TREE_BROADCAST, _lib.OP_TREE_REDUCE,
+                                _lib.OP_ALLGATHER_TEMPORAL])
+def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     """Whatever the collective and the world size, the tuned geometry passes the
     library's own plan check, deals whole channels to the 8 XCDs, fits its
     staging budget and stays inside the wavefront budget."""
     from tests.test_abi import make_op
-    reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
-    threads = common.TUNED_THREADS_REDUCING if reducing else 256
-    slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS)
+    reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_TREE_REDUCE)
+    threads = common.TUNED_THREADS_REDUCING if reducing and op != _lib.OP_TREE_REDUCE else 256
+    slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS,
+                                                row_blocks=row_blocks)
     assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
     multi = op in (_lib.OP_ALLGATHER, _lib.OP_ALLTOALL)
     d = make_op(op=op, world=world, slot_bytes=slot, nslots=nslots, waves_per_channel_group=waves,
