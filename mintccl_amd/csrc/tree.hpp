@@ -92,6 +92,14 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
     const uint64_t flag_hi = (uint64_t)epoch << 32;
     uint32_t credits_seen[kTreeArity] = {0u, 0u};
 
+    // Own rows one block ahead (whole blocks only; the ragged last block of a
+    // row is loaded where it is used): the load from HBM is in flight while
+    // the block before it is polled for, added and sent.
+    const uint32_t nfull = (uint32_t)(row_bytes / kBlockRawLL);
+    const uint32_t last_k = K - 1u;
+    u32x4 ahead = {0u, 0u, 0u, 0u};
+    if (load && (uint32_t)w < nfull) ahead = ll_fetch_raw(in_row, row_bytes, (uint32_t)w, true, m);
+
     uint32_t slot = 0;
     for (uint32_t s = 0; s < a.steps; ++s) {
         const uint32_t tag = (epoch << 20) | (s + 1u);
@@ -111,15 +119,22 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
             if (g >= nblocks) break;
             const uint32_t at = slot * a.slot_bytes + idx * kBlockMsg;
             u32x4 x = {0u, 0u, 0u, 0u};
-            if (load) x = ll_load_raw(in_row, row_bytes, g, m);
+            if (load) x = g < nfull ? ll_arrange(ahead, true, m) : ll_load_raw(in_row, row_bytes, g, m);
             // first poll of every incoming block at once, then the repeats
             u32x4 r[kTreeArity];
             uint32_t pending = 0;
             compiler_fence();
 #pragma unroll
             for (int j = 0; j < kTreeArity; ++j)
-                if (j < nin && !ll_poll<LDCP>(own, at + (uint32_t)j * a.step_msg, tag, m, r[j]))
-                    pending |= 1u << j;
+                if (j < nin) r[j] = ld128<LDCP>(own, at + (uint32_t)j * a.step_msg + m.lane * 16u);
+            // the wave-channel's next block: k + 1 of this step, or block 0 of the next
+            {
+                const uint32_t gn = k < last_k ? g + W : (s + 1u) * a.step_blocks + (uint32_t)w;
+                if (load && gn < nfull) ahead = ll_fetch_raw(in_row, row_bytes, gn, true, m);
+            }
+#pragma unroll
+            for (int j = 0; j < kTreeArity; ++j)
+                if (j < nin && !wave_all(!m.flag_lane || r[j].w == tag)) pending |= 1u << j;
             for (uint32_t spins = 0; pending; ++spins) {
                 if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status))) {
                     report_timeout(a.status, 0, h, w, s);
