@@ -50,12 +50,12 @@ HBM_PEAK_GBPS = 8000.0
 L2_PEAK_GBPS = 128 * 128 * 2.4          # 128 channels x 128 B per clock x 2.4 GHz
 
 # launch geometry used for the headline (the library's tuned default for this
-# collective): 3 slots of 512 KiB per rank, so that all staging of an XCD's
-# channels stays in its 4 MiB L2, 64 wave-channels per (chunk, hop) in thread
+# collective): 3 slots of 448 KiB per rank, so that all staging of an XCD's
+# channels stays in its 4 MiB L2, 56 wave-channels per (chunk, hop) in thread
 # blocks of two, every hop of a channel on one XCD
-BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 3 * 512 * 1024))
+BUFF_BYTES = int(os.getenv("MINTCCL_BENCH_BUFF", 3 * 448 * 1024))
 NSLOTS = int(os.getenv("MINTCCL_BENCH_NSLOTS", 3))
-WAVES_PER_RANK = int(os.getenv("MINTCCL_BENCH_WAVES", 512))
+WAVES_PER_RANK = int(os.getenv("MINTCCL_BENCH_WAVES", 448))
 THREADS = int(os.getenv("MINTCCL_BENCH_THREADS", 128))
 PLACEMENT = int(os.getenv("MINTCCL_BENCH_PLACEMENT", 1))      # 0 spread, 1 local
 CACHE_POLICY = int(os.getenv("MINTCCL_BENCH_CACHE", 2))       # 0 agent, 1 system, 2 XCD-local

@@ -115,13 +115,16 @@ class Timer:
 # (from about 6100 on the grid no longer runs as one wave of blocks and the
 # time jumps by a third).  Everything else - the collectives with a single
 # pipeline (sendrecv, broadcast, reduce) and the reducing ones (reducescatter,
-# allreduce): 3 slots of 512 KiB, 4608 wavefronts; a slot may grow to
-# TUNED_SLOT_BUDGET bytes when there are few hops.  The reducing collectives
+# allreduce): 3 slots of 512 KiB, 4608 wavefronts (reducescatter: 3 slots of
+# 448 KiB, 56 wave-channels per (row, hop) instead of 64: 1.5 - 2 % faster);
+# a slot may grow to TUNED_SLOT_BUDGET bytes when there are few hops.  The
+# reducing collectives
 # run thread blocks of 2 wave-channels (TUNED_THREADS_REDUCING) unless the
 # caller names a block size.  Staging is allocated for TUNED_NSLOTS slots of
 # TUNED_SLOT_BUDGET either way.
 TUNED_TOTAL_WAVES = 4608
 TUNED_SLOT_BLOCKS = 512
+TUNED_SLOT_BLOCKS_REDUCESCATTER = 448
 TUNED_NSLOTS = 3
 TUNED_TOTAL_WAVES_MULTI = 5760
 TUNED_SLOT_BLOCKS_MULTI = 640
@@ -183,7 +186,8 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
     # slots sized per 8 receiving ranks keep the staging of an XCD's channels
     # (slots x receivers / 8) well inside its 4 MiB of L2
     multi = op == _lib.OP_ALLGATHER
-    per8 = TUNED_SLOT_BLOCKS_MULTI if multi else TUNED_SLOT_BLOCKS
+    per8 = TUNED_SLOT_BLOCKS_MULTI if multi else (
+        TUNED_SLOT_BLOCKS_REDUCESCATTER if op == _lib.OP_REDUCESCATTER else TUNED_SLOT_BLOCKS)
     total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
     if fetcher_waves:
         # every thread block carries one more wavefront (it streams own rows

@@ -67,7 +67,7 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
 
 
 def test_headline_geometry():
-    assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 128, 3) == (512 * 1024, 3, 64)
+    assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 128, 3) == (448 * 1024, 3, 56)
     assert common.tuned_geometry(_lib.OP_ALLREDUCE, 8, 0, 128, 3) == (512 * 1024, 3, 32)
     assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
