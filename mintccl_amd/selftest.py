@@ -169,7 +169,11 @@ def reduce() -> bool:
     _run_all(comm, lambda r: op(bufs[r], root, comm))
     if inputs is None:
         return True
-    want = _ring_fold(inputs, ring_of(comm), root)
+    from . import tree
+    if tree.topology_env() == "tree":       # the operator went up the binary tree
+        want = _tree_fold(inputs, tree.nodes(ring_of(comm), root))
+    else:
+        want = _ring_fold(inputs, ring_of(comm), root)
     _order_free_distance(root, bufs[root], inputs)
     return _report(root, bufs[root], want, True)
 

@@ -185,3 +185,20 @@ def test_tree_self_tests_pass(dev, monkeypatch, capsys):
     assert selftest.main("tree_reduce") == 0
     out = capsys.readouterr().out
     assert out.count("equal: True") == 8 + 1 and "equal: False" not in out
+
+
+def test_ring_self_tests_follow_the_topology_switch(dev, monkeypatch, capsys):
+    """With MINTCCL_TOPOLOGY=tree the reduce self-test compares with the tree's
+    order of additions (the operator it runs went up the tree)."""
+    from mintccl_amd import selftest
+    monkeypatch.setenv("MINTCCL_TEST_MODE", "1")
+    monkeypatch.setenv("MINTCCL_TEST_COUNT", str(1 << 18))
+    monkeypatch.setenv("MINTCCL_WORLD_SIZE", "5")
+    monkeypatch.setenv("MINTCCL_TOPOLOGY", "tree")
+    monkeypatch.setenv("MINTCCL_ALLGATHER", "temporal")
+    assert selftest.main("reduce") == 0
+    assert selftest.main("broadcast") == 0
+    assert selftest.main("allgather") == 0
+    out = capsys.readouterr().out
+    assert "equal: False" not in out and out.count("equal: True") == 1 + 5 + 5
+
