@@ -217,6 +217,31 @@ def test_device_epoch_wraps_and_clears(dev):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("world", [3, 6, 7])
+@pytest.mark.parametrize("knobs", [
+    {},
+    {"MINTCCL_PROTOCOL": "simple"},
+    {"MINTCCL_PLACEMENT": "spread", "MINTCCL_CACHE": "agent"},
+    {"MINTCCL_TOPOLOGY": "tree", "MINTCCL_ALLGATHER": "temporal"},
+    {"MINTCCL_ALLREDUCE": "split", "MINTCCL_NSLOTS": "2", "MINTCCL_BUFFSIZE": "262144"},
+    {"MINTCCL_DEVICE_EPOCH": "1", "ROOT_TEMP": "1"},
+])
+def test_self_tests_over_world_sizes_and_knobs(monkeypatch, capsys, world, knobs):
+    """Every operator's self-test under the environment knobs a user can set,
+    on world sizes the other tests do not visit."""
+    from mintccl_amd import selftest
+    monkeypatch.setenv("MINTCCL_TEST_MODE", "1")
+    monkeypatch.setenv("MINTCCL_TEST_COUNT", str((1 << 18) + 8 * world))
+    monkeypatch.setenv("MINTCCL_WORLD_SIZE", str(world))
+    for k, v in knobs.items():
+        monkeypatch.setenv(k, v)
+    assert selftest.main("all") == 0
+    out = capsys.readouterr().out
+    assert "equal: False" not in out
+    assert out.count("equal: True") == 3 + 4 * world + 1 + world + world + 1
+
+
+@pytest.mark.gpu
 def test_captured_collectives_replay(dev):
     """A captured sequence of collectives (epoch in device memory) is replayed
     several times, with eager work and fresh inputs in between; every replay
