@@ -210,12 +210,12 @@ def config4(reps: int) -> None:
                  hbm_bytes=(world + 1) * S, algbw_gbps=round(S / ms / 1e6, 1), ok=ok, grid=comm.last_grid)
 
 
-def config5(reps: int, max_log2: int) -> None:
+def config5(reps: int, max_log2: int, only_log2=()) -> None:
     world = 8
     for name, proto in (("ll128", 0), ("simple", 1)):
         comms = {label: comm_for(world, proto, slots, waves_per_rank=512 if slots else None)
                  for label, slots in geometries("8x512KiB", (8, 512 * 1024))}
-        for log2 in range(9, max_log2 + 1):
+        for log2 in (only_log2 or range(9, max_log2 + 1)):
             shard = 1 << log2
             n = shard // 2
             bufs = []
@@ -424,6 +424,8 @@ def main() -> int:
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
     ap.add_argument("--only", type=int, default=0,
                     help="run one config (2..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring)")
+    ap.add_argument("--shard-log2", default="",
+                    help="config 5: only these shard sizes (log2 of bytes, comma separated)")
     ap.add_argument("--tree-log2", default="10,14,17,20,23,26",
                     help="config 10: log2 of the message sizes (bytes per rank)")
     args = ap.parse_args()
@@ -438,7 +440,8 @@ def main() -> int:
     if args.only in (0, 4):
         config4(reps)
     if args.only in (0, 5):
-        config5(reps, 24 if args.quick else 27)
+        config5(reps, 24 if args.quick else 27,
+                tuple(int(x) for x in args.shard_log2.split(",") if x))
     if args.only in (0, 8):
         allreduce_bench(reps)
     if args.only in (0, 9):
