@@ -118,9 +118,10 @@ class Timer:
 # allreduce): 3 slots of 512 KiB, 4608 wavefronts (reducescatter: 3 slots of
 # 448 KiB, 56 wave-channels per (row, hop) instead of 64: 1.5 - 2 % faster);
 # a slot may grow to TUNED_SLOT_BUDGET bytes when there are few hops.  The
-# reducing collectives
-# run thread blocks of 2 wave-channels (TUNED_THREADS_REDUCING) unless the
-# caller names a block size.  Staging is allocated for TUNED_NSLOTS slots of
+# reducing collectives, sendrecv and alltoall run thread blocks of 2
+# wave-channels (TUNED_THREADS_REDUCING; sendrecv -9 %, alltoall -7 % against
+# blocks of 4; broadcast the same either way, allgather 7 % slower) unless
+# the caller names a block size.  Staging is allocated for TUNED_NSLOTS slots of
 # TUNED_SLOT_BUDGET either way.
 TUNED_TOTAL_WAVES = 4608
 TUNED_SLOT_BLOCKS = 512
@@ -392,7 +393,8 @@ class VirtualComm:
         if self.auto_geometry:
             lds = (self.row_fetch == _lib.FETCH_LDS and d.protocol == _lib.PROTO_LL128
                    and reducing and threads // 64 in (4, 7))
-            if reducing and not lds and not self.threads_explicit:
+            pairs = reducing or op in (_lib.OP_SENDRECV, _lib.OP_ALLTOALL)
+            if pairs and not lds and not self.threads_explicit:
                 threads = TUNED_THREADS_REDUCING
             row = count_bytes
             if op == _lib.OP_ALLREDUCE:

@@ -41,7 +41,9 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     staging budget and stays inside the wavefront budget."""
     from tests.test_abi import make_op
     reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_TREE_REDUCE)
-    threads = common.TUNED_THREADS_REDUCING if reducing and op != _lib.OP_TREE_REDUCE else 256
+    pairs = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE, _lib.OP_SENDRECV,
+                   _lib.OP_ALLTOALL)
+    threads = common.TUNED_THREADS_REDUCING if pairs else 256
     slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS,
                                                 row_blocks=row_blocks)
     assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
