@@ -520,6 +520,14 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             }
         }
         if (timing) { t_poll += wall_clock64() - t1; ++n_groups; }
+        if (PROTO == PROTO_LL128 && q.last && role.recv && lane_id() == 0) {
+            // post_ll128 (protocol.py:183-189): the tags have been tested, so
+            // every line of step s is in registers and the slot is free.  The
+            // post goes out ahead of this group's own stores: the sender's
+            // credit does not queue behind them.
+            if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
+            else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
+        }
         asm volatile("" : "+v"(credit_word));
         if (ask_credit) {
             const uint64_t t0 = timing ? wall_clock64() : 0;
@@ -565,10 +573,9 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             }
         }
         if (q.last) {
-            // post_ll128 (protocol.py:183-189): this wave-channel has taken every
-            // line of step s out of its slot (the loads have returned: their
-            // values were tested / used above).
-            if (role.recv && lane_id() == 0) {
+            // Simple protocol: this wave-channel has taken every line of step s
+            // out of its slot (the stores above carry what the loads returned).
+            if (PROTO == PROTO_SIMPLE && role.recv && lane_id() == 0) {
                 if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(s + 1));
                 else st64_agent(own_tail, flag_hi | (uint64_t)(s + 1));
             }
@@ -660,7 +667,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 if (role.save) store_pad();
                 if (role.send) store_pad();
             }
-            if (role.recv) store_pad();
             compiler_fence();
             if (role.load) fetch_step(1, vv[1]);
             auto whole_step = [&](auto phase) MINT_INLINE_LAMBDA {
@@ -691,6 +697,14 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     }
                 }
                 ++n_groups;
+                if (role.recv) {
+                    // post_ll128 (protocol.py:183-189), as soon as the step is in
+                    // registers and ahead of this step's own stores, so that the
+                    // credit does not queue behind them; every lane stores the
+                    // same word
+                    if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1));
+                    else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1));
+                }
                 if (role.send) {
                     asm volatile("" : "+v"(cw[B]));
                     if (credits_seen < need) {
@@ -722,11 +736,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     if (role.save)
                         ll_save_raw(out_row, row_bytes, step * a.step_blocks + idx, true, m, x);
                     if (role.send) ll_send<STCP>(nxt, send_base + idx * kBlockMsg, x, tag, m);
-                }
-                if (role.recv) {
-                    // post_ll128 (protocol.py:183-189); every lane stores the same word
-                    if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1));
-                    else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1));
                 }
                 compiler_fence();
                 if (role.load) fetch_step(step + 2u, vv[B]);
