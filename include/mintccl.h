@@ -289,8 +289,11 @@ int mint_ring_launch(const mint_ring_op* op, void* stream);
  * bounded waits and the status block).  stats: 0, or - in a library built
  * with -DMINT_RING_STATS only, others refuse it - the device address of
  * (hops + 1) x 8 zeroed uint64 that receive, per position, {groups, re-polls,
- * ticks waiting for credit, ticks polling, ticks total, wavefronts, 0, 0}; a
- * tick is 10 ns.  No counterpart in the reference. */
+ * ticks waiting for credit, ticks polling, ticks total, wavefronts, ticks
+ * waiting for own rows fetched ahead (LL128 copying walks and the walk with
+ * own rows through LDS), ticks issuing a step's loads and stores (LL128
+ * copying walks; the LDS walk: its fetchers' wait for room)}; a tick is
+ * 10 ns.  No counterpart in the reference. */
 typedef struct {
     uint32_t skip_origin;
     uint32_t reserved0;

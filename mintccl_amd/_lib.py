@@ -129,7 +129,8 @@ def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | N
     compilations run side by side and are linked at the end.  ``defines``
     (``-DMINT_RING_STATS``: wait accounting per ring position,
     ``-DMINT_EARLY_POLL_ALL``: the adding kernels poll a step ahead like the
-    copying ones) and ``so_path`` make a diagnostic build beside the product's;
+    copying ones, ``-DMINT_ROW_NOLOAD``: whole blocks of own rows are not
+    loaded - wrong results, for timing a collective without its HBM reads) and ``so_path`` make a diagnostic build beside the product's;
     ``MINTCCL_LIBRARY`` loads it."""
     out = so_path or os.path.join(_PKG, "libmintccl.so")
     build_dir = BUILD_DIR if so_path is None else out + ".objs"

@@ -240,6 +240,13 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     a.stats = nullptr;
 #endif
     a.placement = op->placement;
+    {
+        // (MI355X: 256 CUs in 8 XCDs; only a matter of speed)
+        constexpr int kCusPerXcd = 32;
+        const int npos = a.hops + 1;
+        a.seat_turn = (over_tree(op->op) || temporal) && kCusPerXcd % npos == 0
+                          ? (uint32_t)(kCusPerXcd / npos) : 0u;
+    }
 
     const int waves_per_block = (int)op->threads_per_block / 64;
     plan->threads = (int)op->threads_per_block;

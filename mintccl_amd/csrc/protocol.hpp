@@ -114,8 +114,14 @@ __device__ __forceinline__ u32x4 ll_fetch_raw(const uint8_t* row, uint64_t row_b
         // flag lanes start 4 bytes early so that all 64 lanes issue one
         // 16-byte load that stays inside the block
         const uint32_t off = m.flag_lane ? m.raw_off - 4u : m.raw_off;
+#ifdef MINT_ROW_NOLOAD
+        // diagnostic build: no load, the block's number instead of its bytes
+        // (what a collective costs without its reads of the rows from HBM)
+        return u32x4{g, off, 3u, 4u};
+#else
         return __builtin_nontemporal_load(
             (MINT_GLOBAL const u32x4_a1*)(row + base + off));
+#endif
     }
     return load_guarded(row, base + m.raw_off, m.raw_len, row_bytes);
 }

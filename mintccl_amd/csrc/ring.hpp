@@ -74,6 +74,7 @@ struct RingArgs {
     const uint32_t* epoch_word;           // optional: take the epoch from device memory instead
     uint64_t* status;
     uint32_t skip_origin;
+    uint32_t seat_turn;                   // local placement: channels after which the positions turn by two (0: never)
     uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
     uint32_t fetch_depth;                 // own rows through LDS: groups of LDS per wave-channel
 };
@@ -360,7 +361,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
 #else
     constexpr bool timing = false;
 #endif
-    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0, t_lds = 0;
+    uint64_t t_credit = 0, t_poll = 0, n_repoll = 0, n_groups = 0, t_lds = 0, t_issue = 0;
     const uint64_t t_begin = timing ? wall_clock64() : 0;
 
     // Group = U blocks of this wave-channel inside one step
@@ -619,7 +620,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // stored by all lanes, fetch addresses are clamped), a wave that gives up
     // ends on the spot instead of leaving the loop, and the prologue issues
     // exactly the queue a later step finds (stand-ins for the stores go to an
-    // unused part of this wave-channel's own credit line).
+    // unused part of a credit line of this wave-channel: the one it looks at
+    // when it sends, else its own).
 #ifdef MINT_EARLY_POLL_ALL
     if constexpr (PROTO == PROTO_LL128) {
 #else
@@ -648,7 +650,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     x[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
                 }
             };
-            uint64_t* const pad = own_tail + 8;
+            // (an origin need not have staging of its own)
+            uint64_t* const pad = role.send ? nxt_tail + 8 : own_tail + 8;
             auto store_pad = [&]() MINT_INLINE_LAMBDA {
                 if (STCP == CP_NONE) st64_local(pad, 0ull);
                 else st64_agent(pad, 0ull);
@@ -676,6 +679,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 const uint32_t need = step >= a.nslots ? step - a.nslots + 1 : 0;
                 const uint32_t recv_base = slot * a.slot_bytes + share_recv * a.step_msg;
                 const uint32_t send_base = slot * a.slot_bytes + share_send * a.step_msg;
+                const uint64_t t1 = timing ? wall_clock64() : 0;
                 if (role.recv) {
                     uint32_t pending = 0;
 #pragma unroll
@@ -697,6 +701,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     }
                 }
                 ++n_groups;
+                if (timing) t_poll += wall_clock64() - t1;
                 if (role.recv) {
                     // post_ll128 (protocol.py:183-189), as soon as the step is in
                     // registers and ahead of this step's own stores, so that the
@@ -705,7 +710,15 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1));
                     else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1));
                 }
+                if (timing && role.load) {
+                    // how long the own rows fetched two steps ago still take to arrive
+                    const uint64_t t0 = wall_clock64();
+#pragma unroll
+                    for (int u = 0; u < U; ++u) asm volatile("" : "+v"(vv[B][u]));
+                    t_lds += wall_clock64() - t0;
+                }
                 if (role.send) {
+                    const uint64_t t0 = timing ? wall_clock64() : 0;
                     asm volatile("" : "+v"(cw[B]));
                     if (credits_seen < need) {
                         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(cw[B] >> 32));
@@ -715,9 +728,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                                              a.status))
                             give_up();
                     }
+                    if (timing) t_credit += wall_clock64() - t0;
                 }
                 // the next step's credit word and first poll go out ahead of this step's stores
                 compiler_fence();
+                const uint64_t t2 = timing ? wall_clock64() : 0;
                 if (role.send) cw[B1] = ld64_agent(nxt_tail);
                 if (role.recv) poll_step(next_slot, rr[B1]);
                 compiler_fence();
@@ -739,6 +754,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 }
                 compiler_fence();
                 if (role.load) fetch_step(step + 2u, vv[B]);
+                if (timing) {
+                    // how long the step's loads and stores took to issue
+                    compiler_fence();
+                    t_issue += wall_clock64() - t2;
+                }
                 slot = next_slot;
                 ++step;
             };
@@ -776,6 +796,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         atomicAdd(st + 4, (unsigned long long)(wall_clock64() - t_begin));
         atomicAdd(st + 5, 1ull);
         atomicAdd(st + 6, (unsigned long long)t_lds);
+        atomicAdd(st + 7, (unsigned long long)t_issue);
     }
 }
 
@@ -813,15 +834,27 @@ __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib) {
         // how far along that XCD's list of work it is: XCD d takes the
         // channels c with c % 8 == d and its blocks walk through the
         // positions of one channel after the other.  A channel's whole ring
-        // then shares one L2 by construction, is dispatched together, and
-        // every CU hosts a mix of positions.
+        // then shares one L2 by construction and is dispatched together.
         const int xcd = xcc_id(), y = x / kXcds;
         if (xcd >= kXcds) {
             report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
             return st;
         }
-        st.h = y % npos;
-        c = (y / npos) * kXcds + xcd;
+        //
+        // An XCD hands its blocks to its CUs in turn, so with h = y % npos and a
+        // position count that divides the CUs of an XCD (8 ranks) every CU
+        // holds blocks of one position only: the positions that load from HBM
+        // sit on CUs of their own and the polls of the others, answered by
+        // the L2, never queue behind a load from HBM in a CU's memory
+        // pipeline.  The ring walks are fastest that way (an allgather whose
+        // CUs hold a mix of positions takes 4 - 10 % longer).  The tree and
+        // the temporal allgather, where the loading position of a wave-channel
+        // is one of few or changes from phase to phase, gain 6 - 10 % from a
+        // mix: seat_turn turns the positions by two after every round over the
+        // CUs.
+        const int q = y / npos;
+                st.h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
+        c = q * kXcds + xcd;
     } else {
         st.h = x % npos;
         c = x / npos;

@@ -245,6 +245,37 @@ def test_broadcast_bytes(dev, world, nbytes, proto):
         assert torch.equal(b.cpu(), host[root])
 
 
+@pytest.mark.parametrize("proto", [0, 1])
+@pytest.mark.parametrize("policy", [(0, 0), (1, 2)])
+def test_an_origin_needs_no_staging(dev, proto, policy):
+    """The root of a broadcast and the source of a sendrecv receive nothing:
+    the library accepts a descriptor without staging for them and touches none
+    (whole steps, a ragged last step and a message shorter than a block)."""
+    from mintccl_amd import _lib
+    world, root = 4, 3
+    comm = make_comm(world, protocol=proto, placement=policy[0], cache_policy=policy[1])
+    ring_order = list(range(world)) + [0]
+    for nbytes in ((3 << 20) + 5, 100, 960 * 64 * 8):
+        g = torch.Generator().manual_seed(nbytes)
+        host = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g) for _ in range(world)]
+        bufs = [h.to(dev) for h in host]
+        ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+        d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, nbytes, {root: ptrs[root]},
+                         {r: p for r, p in ptrs.items() if r != root}, ring_order, root=root)
+        d.staging[root] = 0
+        comm.launch(d)
+        comm.check()
+        for b in bufs:
+            assert torch.equal(b.cpu(), host[root])
+        bufs = [h.to(dev) for h in host]
+        d = comm.make_op(_lib.OP_SENDRECV, _lib.BYTES, nbytes, {2: bufs[2].data_ptr()},
+                         {1: bufs[1].data_ptr()}, [2, 1], route_len=2)
+        d.staging[2] = 0
+        comm.launch(d)
+        comm.check()
+        assert torch.equal(bufs[1].cpu(), host[2]) and torch.equal(bufs[0].cpu(), host[0])
+
+
 @pytest.mark.parametrize("world", WORLDS)
 @pytest.mark.parametrize("n", [8, 480, 488, 65536])
 @pytest.mark.parametrize("proto", [0, 1])
