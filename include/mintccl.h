@@ -178,6 +178,19 @@ typedef struct {
                               captured into a HIP graph and replayed: put a
                               mint_epoch_advance on the same word in front of
                               every launch. */
+    uint32_t origin_cus;   /* 0, or of the 32 compute units of an XCD so many
+                              hold nothing but origins (the positions that
+                              read the caller's rows from HBM): BROADCAST and
+                              ALLGATHER of 4 ranks or more under
+                              MINT_PLACE_LOCAL with at least 64 thread blocks
+                              per position, below 32; ignored elsewhere, and
+                              where the larger grid it needs (blocks with
+                              nothing to do fill the rounds) would not be
+                              resident.  A matter of speed only: a compute
+                              unit keeps a bounded number of loads in flight,
+                              and an eighth of them cannot feed an 8-rank
+                              ring.  No counterpart in the reference. */
+    uint32_t reserved1;    /* 0 */
 } mint_ring_op;
 
 int mint_version(void);

@@ -66,6 +66,7 @@ class RingOp(ctypes.Structure):
         ("row_fetch", ctypes.c_int32), ("credit_offset", ctypes.c_uint32),
         ("total_bytes", ctypes.c_uint64),
         ("epoch_ptr", ctypes.c_uint64),
+        ("origin_cus", ctypes.c_uint32), ("reserved1", ctypes.c_uint32),
     ]
 
 

@@ -110,13 +110,12 @@ class Timer:
 
 
 # Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
-# step.  The copying collectives with one pipeline per rank (allgather,
-# alltoall): 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in all
-# (from about 6100 on the grid no longer runs as one wave of blocks and the
-# time jumps by a third).  Everything else - the collectives with a single
-# pipeline (sendrecv, broadcast, reduce) and the reducing ones (reducescatter,
-# allreduce): 3 slots of 512 KiB, 4608 wavefronts (reducescatter: 3 slots of
-# 448 KiB, 56 wave-channels per (row, hop) instead of 64: 1.5 - 2 % faster);
+# step.  Alltoall: 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in
+# all (from about 6100 on the grid no longer runs as one wave of blocks and the
+# time jumps by a third).  Everything else: 3 slots of 512 KiB, 4608
+# wavefronts (reducescatter: 3 slots of 448 KiB, 56 wave-channels per
+# (row, hop) instead of 64: 1.5 - 2 % faster; broadcast and allgather with CUs
+# set apart for their origins, tuned_origin_cus);
 # a slot may grow to TUNED_SLOT_BUDGET bytes when there are few hops.  The
 # reducing collectives, sendrecv and alltoall run thread blocks of 2
 # wave-channels (TUNED_THREADS_REDUCING; sendrecv -9 %, alltoall -7 % against
@@ -186,19 +185,39 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         npos = (npos + 1) // 2    # `pipes` already counts both phases
     # slots sized per 8 receiving ranks keep the staging of an XCD's channels
     # (slots x receivers / 8) well inside its 4 MiB of L2
-    multi = op == _lib.OP_ALLGATHER
-    per8 = TUNED_SLOT_BLOCKS_MULTI if multi else (
-        TUNED_SLOT_BLOCKS_REDUCESCATTER if op == _lib.OP_REDUCESCATTER else TUNED_SLOT_BLOCKS)
-    total = TUNED_TOTAL_WAVES_MULTI if multi else TUNED_TOTAL_WAVES
+    per8 = TUNED_SLOT_BLOCKS_REDUCESCATTER if op == _lib.OP_REDUCESCATTER else TUNED_SLOT_BLOCKS
+    total = TUNED_TOTAL_WAVES
     if fetcher_waves:
         # every thread block carries one more wavefront (it streams own rows
         # into LDS) and a CU takes whole blocks: 24 wavefronts per CU, 256 CUs
         total = (24 // (wpb + 1)) * 256 * wpb
-    nslots = min(max_nslots, TUNED_NSLOTS_MULTI) if multi else max_nslots
+    nslots = max_nslots
     slot_blocks = min(per8 * max(1, 8 // receivers), total // npos, TUNED_SLOT_BUDGET // 1024)
     granule = wpb * (8 // math.gcd(real_pipes, 8))
     waves = max(granule, slot_blocks // pipes // granule * granule)
     return fit(pipes, nslots, waves, granule)
+
+
+def tuned_origin_cus(op: int, world: int, channels: int, waves_per_block: int) -> int:
+    """Of the 32 CUs of an XCD, how many the origins of a ring broadcast or
+    allgather get to themselves; ``channels`` = thread blocks per position of
+    the launch (the library ignores the number for small grids and other
+    collectives).  A CU keeps about 26 KB of loads in flight and a load from
+    HBM takes 2.5 us while the collective's stores saturate it, so the
+    origins' natural share of the CUs - one position in ``world`` - delivers
+    too little: measured best at 8 ranks is 9 of 32 (allgather of 8 x 128 MiB
+    3.38 -> 2.57 ms, broadcast of 64 MiB 0.237 -> 0.171 ms), 2.25 times the
+    natural share, which is what other ring lengths aim for.  The grid is
+    filled up to whole rounds over the CUs and has to stay resident (24
+    wavefronts per CU): the largest count up to the aim that fits."""
+    if op not in (_lib.OP_BROADCAST, _lib.OP_ALLGATHER) or world < 4 or channels % 8:
+        return 0
+    groups, rounds_max = channels // 8, 24 // max(1, waves_per_block)
+    for n in range(max(1, min(16, round(72 / world))), 0, -1):
+        rounds = max(-(-groups // n), -(-(world - 1) * groups // (32 - n)))
+        if rounds <= rounds_max:
+            return n
+    return 0
 
 
 _XCDS: dict[int, int] = {}
@@ -239,7 +258,8 @@ class VirtualComm:
                  protocol: int | None = None, placement: int | None = None,
                  waves_per_rank: int | None = None, threads_per_block: int | None = None,
                  cache_policy: int | None = None, spin_budget: int = 0,
-                 device_epoch: bool | None = None, row_fetch: int | None = None) -> None:
+                 device_epoch: bool | None = None, row_fetch: int | None = None,
+                 origin_cus: int | None = None) -> None:
         self.world_size = world_size if world_size is not None else world_size_env()
         if not 1 <= self.world_size <= _lib.MAX_RANKS:
             raise ValueError(f"world_size must be 1..{_lib.MAX_RANKS}")
@@ -285,6 +305,11 @@ class VirtualComm:
             raise ValueError("the XCD-local cache policy needs the local placement")
         self.spin_budget = spin_budget
         self.row_fetch = row_fetch if row_fetch is not None else row_fetch_env()
+        # CUs per XCD set apart for the origins of a ring broadcast / allgather:
+        # an argument, MINTCCL_ORIGIN_CUS (0: none), or the tuned count
+        if origin_cus is None and os.getenv("MINTCCL_ORIGIN_CUS"):
+            origin_cus = _env_int("MINTCCL_ORIGIN_CUS", 0)
+        self.origin_cus = origin_cus
         self._lib = _lib.lib()          # fails loudly if the extension is missing
         # slots + credit words (never more than slot_bytes / 4), zeroed: flag 0
         # and credit 0 mean "nothing yet" (2_sendrecv_indirect.py:59-60).
@@ -430,6 +455,10 @@ class VirtualComm:
             if channels % 8:
                 d.placement = _lib.PLACE_SPREAD
                 d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy
+            elif self.origin_cus is not None:
+                d.origin_cus = self.origin_cus
+            elif self.auto_geometry:
+                d.origin_cus = tuned_origin_cus(op, self.world_size, channels, wpb)
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
         # test hooks travel beside the descriptor (mint_ring_launch_debug)

@@ -241,8 +241,6 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
 #endif
     a.placement = op->placement;
     {
-        // (MI355X: 256 CUs in 8 XCDs; only a matter of speed)
-        constexpr int kCusPerXcd = 32;
         const int npos = a.hops + 1;
         a.seat_turn = (over_tree(op->op) || temporal) && kCusPerXcd % npos == 0
                           ? (uint32_t)(kCusPerXcd / npos) : 0u;
@@ -265,6 +263,24 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // the XCD-local mapping deals whole channels to XCDs
     if (op->placement == MINT_PLACE_LOCAL && (a.pipes * a.blocks_per_group) % kXcds)
         return MINT_ERR_GEOMETRY;
+    // Large ring broadcasts and allgathers under the local placement: origins
+    // on CUs which they have to themselves, as many as the caller names
+    // (take_seat); the grid grows by the blocks that find nothing to do.
+    a.origin_cus = 0;
+    {
+        const int npos = a.hops + 1, groups = a.pipes * a.blocks_per_group / kXcds;
+        const int origin_cus = (int)op->origin_cus;
+        if (origin_cus >= kCusPerXcd || op->reserved1) return MINT_ERR_ARG;
+        plan->blocks_plain = plan->blocks;
+        if (op->placement == MINT_PLACE_LOCAL && origin_cus > 0 && npos >= 4 && groups >= 8 &&
+            (op->op == MINT_OP_BROADCAST || op->op == MINT_OP_ALLGATHER)) {
+            const int others = kCusPerXcd - origin_cus;
+            const int r0 = (groups + origin_cus - 1) / origin_cus;
+            const int r1 = ((npos - 1) * groups + others - 1) / others;
+            a.origin_cus = (uint32_t)origin_cus;
+            plan->blocks = kXcds * kCusPerXcd * (r0 > r1 ? r0 : r1);
+        }
+    }
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
     plan->staging_need = (size_t)a.credit_off + (size_t)a.shares * (size_t)a.waves * kCreditStride;
     // The credit words lie behind the slots: a buffer that only holds the

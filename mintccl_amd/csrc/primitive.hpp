@@ -98,6 +98,34 @@ __device__ __forceinline__ void st64_agent(uint64_t* p, uint64_t v) {
 __device__ __forceinline__ void st64_local(uint64_t* p, uint64_t v) {
     __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
 }
+// A 64-bit word read through the scalar unit, past the scalar cache (glc), from
+// the L2 of the XCD the wave runs on.  Scalar loads count on lgkmcnt, not on
+// vmcnt: a wave can look at a word this way while vector loads of its own are
+// in flight, where a vector load of the word would only come back after all of
+// them (vector loads return in issue order).  Only for words that were stored
+// into this XCD's L2 (the XCD-local staging policy).
+__device__ __forceinline__ uint64_t ld64_scalar(const uint64_t* p) {
+    // The address is the same in every lane; the compiler is told so.
+    // (readfirstlane returns int: through uint32_t, or the low half would be
+    // sign-extended over the high one.)
+    const uint64_t a = (uint64_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    const uint64_t ua = (uint64_t)lo | ((uint64_t)hi << 32);
+    uint64_t v;
+    asm volatile("s_load_dwordx2 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)"
+                 : "=s"(v) : "s"(ua) : "memory");
+    return v;
+}
+// A 32-bit word at agent scope, loaded and waited for inside one asm statement:
+// the compiler's count of outstanding vector-memory operations is left as it
+// was (it then waits for at most as much as it would have).
+__device__ __forceinline__ uint32_t ld32_agent_apart(const void* p) {
+    uint32_t v;
+    asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
 // Release for data that was stored with scope bits (write-through) or, for the
 // XCD-local policy, into the L2 both sides share: once the wave's stores are
 // acknowledged they are visible to every load that skips the L1, so waiting

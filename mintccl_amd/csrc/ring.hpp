@@ -75,6 +75,7 @@ struct RingArgs {
     uint64_t* status;
     uint32_t skip_origin;
     uint32_t seat_turn;                   // local placement: channels after which the positions turn by two (0: never)
+    uint32_t origin_cus;                  // local placement: of the 32 CUs of an XCD, so many hold origins only (0: the plain order)
     uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
     uint32_t fetch_depth;                 // own rows through LDS: groups of LDS per wave-channel
 };
@@ -622,12 +623,120 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // exactly the queue a later step finds (stand-ins for the stores go to an
     // unused part of a credit line of this wave-channel: the one it looks at
     // when it sends, else its own).
+    //
+    // An origin of a copying collective (it loads rows and sends them, and
+    // receives nothing) has its own loop under the XCD-local policy.  Its
+    // only vector loads are the row fetches; the one word it has to look at,
+    // the credit, it reads through the scalar unit, which counts apart.  So
+    // the fetches run kOriginDepth steps ahead and a wait for the oldest
+    // leaves the younger ones in flight: a load from HBM takes 2.5 us under a
+    // collective's stores, twice a step.
+    constexpr int kOriginDepth = 4;
+    constexpr bool kDeepOrigin = PROTO == PROTO_LL128 && DT == DT_BYTES && STCP == CP_NONE &&
+                                 RoleT::load && RoleT::send && !RoleT::recv && !RoleT::save &&
+                                 U <= 2;
+    // (Only where CUs are set apart for the origins: an origin that shares
+    // its CU's memory pipeline gains nothing from more loads in flight -
+    // sendrecv and alltoall take 3 - 7 % longer with this loop.)
+    bool origin_done = false;
+    if constexpr (kDeepOrigin) {
+      if (a.origin_cus && K == (uint32_t)U && ngroups) {
+        origin_done = true;
+        const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
+        uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
+        if (whole_steps > a.steps) whole_steps = a.steps;
+        if (whole_steps) {
+            u32x4 vv[kOriginDepth][U];
+            uint32_t step = 0, slot = 0;
+            auto fetch_step = [&](uint32_t of_step, u32x4 (&x)[U]) MINT_INLINE_LAMBDA {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t g = of_step * a.step_blocks + (uint32_t)u * W + (uint32_t)w;
+                    g = g < nfull ? g : nfull - 1u;      // beyond the whole blocks: any valid address
+                    x[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
+                }
+            };
+            // The queue a later step finds when it waits for its rows: per step
+            // fetched ahead, U sends and the fetch.  The prologue issues the same
+            // (the compiler takes the smaller count where paths meet); stand-ins
+            // for the sends go to an unused part of the credit line this
+            // wave-channel looks at.
+            uint64_t* const pad = nxt_tail + 8;
+            fetch_step(0u, vv[0]);
+#pragma unroll
+            for (int d = 1; d < kOriginDepth; ++d) {
+                compiler_fence();
+#pragma unroll
+                for (int u = 0; u < U; ++u) st64_local(pad, 0ull);
+                compiler_fence();
+                fetch_step((uint32_t)d, vv[d]);
+            }
+            auto origin_step = [&](auto phase) MINT_INLINE_LAMBDA {
+                constexpr int B = decltype(phase)::value;
+                const uint32_t tag = (epoch << 20) | (step + 1u);
+                const uint32_t need = step >= a.nslots ? step - a.nslots + 1 : 0;
+                const uint32_t send_base = slot * a.slot_bytes + share_send * a.step_msg;
+                // wait_ll128 (protocol.py:161-180)
+                const uint64_t t0 = timing ? wall_clock64() : 0;
+                for (uint32_t spins = 0; credits_seen < need; ++spins) {
+                    const uint64_t cw = ld64_scalar(nxt_tail);
+                    if ((uint32_t)(cw >> 32) == epoch && (uint32_t)cw >= need) {
+                        credits_seen = (uint32_t)cw;
+                        break;
+                    }
+                    if (spins >= a.spin_budget ||
+                        ((spins & 63u) == 63u &&
+                         __builtin_amdgcn_readfirstlane(ld32_agent_apart(a.status + 3)) != 0u)) {
+                        report_timeout(a.status, p, h, w, step);
+                        __builtin_amdgcn_endpgm();
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                if (timing) {
+                    const uint64_t t1 = wall_clock64();
+                    t_credit += t1 - t0;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) asm volatile("" : "+v"(vv[B][u]));
+                    t_lds += wall_clock64() - t1;
+                }
+                ++n_groups;
+                const uint64_t t2 = timing ? wall_clock64() : 0;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const uint32_t idx = (uint32_t)u * W + (uint32_t)w;
+                    ll_send<STCP>(nxt, send_base + idx * kBlockMsg, ll_arrange(vv[B][u], true, m), tag, m);
+                }
+                compiler_fence();
+                fetch_step(step + (uint32_t)kOriginDepth, vv[B]);
+                if (timing) {
+                    compiler_fence();
+                    t_issue += wall_clock64() - t2;
+                }
+                slot = slot + 1 == a.nslots ? 0 : slot + 1;
+                ++step;
+            };
+            static_assert(kOriginDepth == 4, "the loop below is unrolled by the depth");
+            while (step < whole_steps) {
+                origin_step(std::integral_constant<int, 0>{});
+                if (step >= whole_steps) break;
+                origin_step(std::integral_constant<int, 1>{});
+                if (step >= whole_steps) break;
+                origin_step(std::integral_constant<int, 2>{});
+                if (step >= whole_steps) break;
+                origin_step(std::integral_constant<int, 3>{});
+            }
+            q.step = step; q.slot = slot; q.k0 = 0;
+            q.fill(geom);
+            n = step;
+        }
+      }
+    }
 #ifdef MINT_EARLY_POLL_ALL
     if constexpr (PROTO == PROTO_LL128) {
 #else
     if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
 #endif
-      if (K == (uint32_t)U && ngroups) {
+      if (!origin_done && K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
         uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
         if (whole_steps > a.steps) whole_steps = a.steps;
@@ -802,6 +911,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
 
 // Which (pipeline, position, wave-channel) a wavefront serves.  `wpb` =
 // wave-channels per thread block, `wib` = this wavefront's index among them.
+constexpr int kCusPerXcd = 32;      // MI355X: 256 CUs in 8 XCDs (a matter of speed only)
 struct Seat {
     int p, h, gw, w;
     bool ok;
@@ -852,8 +962,33 @@ __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib) {
         // is one of few or changes from phase to phase, gain 6 - 10 % from a
         // mix: seat_turn turns the positions by two after every round over the
         // CUs.
-        const int q = y / npos;
-                st.h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
+        int q = y / npos;
+        st.h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
+        if (a.origin_cus) {
+            // Origins on CUs of their own, and on more of them than their share
+            // of the blocks: the XCD's blocks are taken in rounds of one block
+            // per CU; in every round origin_cus of the CUs take an origin, the
+            // others take the receiving positions of the channels in turn.
+            // Blocks left over in either list have nothing to do.  (What a
+            // CU's memory pipeline keeps in flight is bounded, about 26 KB;
+            // loads from HBM under a collective's stores take 2.5 us, so a CU
+            // full of origins delivers 10 GB/s and an eighth of the CUs cannot
+            // feed the rest: allgather 8 x 128 MiB 3.4 ms, 1.9 ms without its
+            // loads.)
+            const int round = y / kCusPerXcd, j = y % kCusPerXcd, o = (int)a.origin_cus;
+            const int groups = a.pipes * a.blocks_per_group / kXcds;
+            // the origins' CUs lie evenly among the 32: `before` of them below CU j
+            const int before = j * o / kCusPerXcd;
+            if ((j + 1) * o / kCusPerXcd > before) {
+                q = round * o + before;
+                st.h = 0;
+            } else {
+                const int r = round * (kCusPerXcd - o) + (j - before);
+                q = r / (npos - 1);
+                st.h = 1 + r % (npos - 1);
+            }
+            if (q >= groups) return st;
+        }
         c = q * kXcds + xcd;
     } else {
         st.h = x % npos;

@@ -94,7 +94,15 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
     }
     int ncu = cus.load(std::memory_order_relaxed);
     if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
+    if (plan.blocks > per_cu * ncu) {
+        // CUs set apart for origins need a larger grid: without, if that fits
+        if (!plan.args.origin_cus || plan.blocks_plain > per_cu * ncu) return MINT_ERR_RESIDENCY;
+        RingArgs plain = plan.args;
+        plain.origin_cus = 0;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks_plain), dim3((unsigned)plan.threads),
+                           0, stream, plain);
+        return launch_status();
+    }
     hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
                        plan.args);
     return launch_status();

@@ -13,6 +13,7 @@ namespace mint {
 struct Plan {
     RingArgs args;
     int blocks, threads, unroll;
+    int blocks_plain;         // the grid without CUs set apart for origins (args.origin_cus)
     size_t staging_need;      // bytes of staging per rank: slots + credit words
     bool empty;
     bool lds;                 // own rows through LDS: `threads` counts the wave-channels'

@@ -159,9 +159,36 @@ def test_plan_geometry_without_a_gpu():
     (dict(op=_lib.OP_ALLREDUCE, waves_per_channel_group=16, total_bytes=4096), _lib.ERR_ARG),
     (dict(count_bytes=(1 << 20) + 1, row_stride=1 << 21), _lib.ERR_ARG),
     (dict(slot_bytes=1 << 30, nslots=8), _lib.ERR_TOO_LARGE),
+    (dict(origin_cus=32), _lib.ERR_ARG), (dict(reserved1=1), _lib.ERR_ARG),
 ])
 def test_plan_rejects_bad_descriptors(kw, err):
     assert _lib.lib().mint_ring_grid_blocks(make_op(**kw)) == err
+
+
+def test_compute_units_set_apart_for_origins_grow_the_grid():
+    """origin_cus: the blocks of an XCD are taken in rounds of 32; in every
+    round so many take an origin, the others the receiving positions; the grid
+    is whole rounds.  Only large ring broadcasts / allgathers under the local
+    placement; ignored elsewhere."""
+    L = _lib.lib()
+    big = dict(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES, placement=1, cache_policy=2,
+               slot_bytes=512 << 10, nslots=3, waves_per_channel_group=64)
+    assert L.mint_ring_grid_blocks(make_op(**big)) == 8 * 8 * 16                   # 4 rounds
+    # 16 channels per XCD: 16 origins over 9 CUs (2 rounds), 112 receivers over 23 (5 rounds)
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **big)) == 8 * 32 * 5
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=4, **big)) == 8 * 32 * 4     # the natural share
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=16, **big)) == 8 * 32 * 7
+    bc = dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, cache_policy=2,
+              slot_bytes=512 << 10, nslots=3, waves_per_channel_group=512)
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **bc)) == 8 * 32 * 5
+    # ignored: small grids, the spread placement, other collectives, short rings
+    small = dict(big, waves_per_channel_group=16, slot_bytes=128 << 10)
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **small)) == 8 * 8 * 4
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **dict(big, placement=0, cache_policy=0))) == 8 * 8 * 16
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, placement=1, waves_per_channel_group=64)) == 8 * 9 * 16
+    two = make_op(origin_cus=9, world=2, **dict(big, slot_bytes=512 << 10, waves_per_channel_group=256))
+    two.ring[2] = 0
+    assert L.mint_ring_grid_blocks(two) == 2 * 2 * 64
 
 
 def test_plan_rejects_bad_buffers_and_rings():

@@ -47,10 +47,13 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS,
                                                 row_blocks=row_blocks)
     assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
-    multi = op in (_lib.OP_ALLGATHER, _lib.OP_ALLTOALL)
+    multi = op == _lib.OP_ALLTOALL
     d = make_op(op=op, world=world, slot_bytes=slot, nslots=nslots, waves_per_channel_group=waves,
                 placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2, threads_per_block=threads,
                 dtype=_lib.F16 if reducing else _lib.BYTES)
+    pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
+    d.origin_cus = common.tuned_origin_cus(op, world, pipes * -(-waves // (threads // 64)),
+                                           threads // 64)
     if op == _lib.OP_ALLTOALL:
         for r in range(8):
             d.output[r] = 0x40000000 + r * 0x1000000
@@ -64,20 +67,26 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     blocks = _lib.lib().mint_ring_grid_blocks(d)
     assert blocks > 0, blocks
     assert blocks % 8 == 0
-    assert blocks * (threads // 64) <= (common.TUNED_TOTAL_WAVES_MULTI if multi
-                                        else common.TUNED_TOTAL_WAVES)
+    # (CUs set apart for origins fill the grid up to whole rounds over the 256
+    # CUs, at most 24 wavefronts each)
+    budget = common.TUNED_TOTAL_WAVES_MULTI if multi else common.TUNED_TOTAL_WAVES
+    assert blocks * (threads // 64) <= (24 * 256 if d.origin_cus else budget)
+    d.origin_cus = 0
+    assert 0 < _lib.lib().mint_ring_grid_blocks(d) <= blocks
+    assert _lib.lib().mint_ring_grid_blocks(d) * (threads // 64) <= budget
 
 
 def test_headline_geometry():
     assert common.tuned_geometry(_lib.OP_REDUCESCATTER, 8, 0, 128, 3) == (448 * 1024, 3, 56)
     assert common.tuned_geometry(_lib.OP_ALLREDUCE, 8, 0, 128, 3) == (512 * 1024, 3, 32)
-    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (640 * 1024, 2, 80)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (512 * 1024, 3, 64)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
     # a small message takes a small grid: the wave-channels are capped at the
     # blocks of one row, in whole thread blocks that the 8 XCDs divide
-    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=1) == (32 * 1024, 2, 4)
-    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=69) == (576 * 1024, 2, 72)
-    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=10 ** 6) == (640 * 1024, 2, 80)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=1) == (32 * 1024, 3, 4)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=61) == (512 * 1024, 3, 64)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=53) == (448 * 1024, 3, 56)
+    assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=10 ** 6) == (512 * 1024, 3, 64)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3, row_blocks=5) == (32 * 1024, 3, 32)
     assert common.tuned_geometry(_lib.OP_TREE_REDUCE, 8, 0, 256, 3, row_blocks=5) == (2 * 32 * 1024, 3, 32)
     assert common.tuned_geometry(_lib.OP_TREE_REDUCE, 8, 0, 256, 3) == (2 * 512 * 1024, 3, 512)
