@@ -180,10 +180,10 @@ typedef struct {
                               every launch. */
     uint32_t origin_cus;   /* 0, or of the 32 compute units of an XCD so many
                               hold nothing but origins (the positions that
-                              read the caller's rows from HBM): BROADCAST and
-                              ALLGATHER of 4 ranks or more under
-                              MINT_PLACE_LOCAL with at least 64 thread blocks
-                              per position, below 32; ignored elsewhere, and
+                              read the caller's rows from HBM): SENDRECV,
+                              BROADCAST and ALLGATHER under MINT_PLACE_LOCAL
+                              with at least 64 thread blocks per position,
+                              below 32; ignored elsewhere, and
                               where the larger grid it needs (blocks with
                               nothing to do fill the rounds) would not be
                               resident.  A matter of speed only: a compute

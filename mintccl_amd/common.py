@@ -131,6 +131,8 @@ TUNED_SLOT_BLOCKS_MULTI = 640
 TUNED_NSLOTS_MULTI = 2
 TUNED_SLOT_BUDGET = 2304 * 1024
 TUNED_THREADS_REDUCING = 128
+TUNED_SENDRECV_SLOT_BLOCKS = 1536
+TUNED_SENDRECV_NSLOTS = 4
 
 
 class RingTimeout(RuntimeError):
@@ -144,7 +146,7 @@ class PlacementError(RuntimeError):
 
 def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
                    max_nslots: int, fetcher_waves: bool = False,
-                   row_blocks: int | None = None) -> tuple[int, int, int]:
+                   row_blocks: int | None = None, ll128: bool = True) -> tuple[int, int, int]:
     """(slot_bytes, nslots, wave-channels per (pipeline, hop)) of the tuned
     geometry for one collective: the wavefront budget spread over the
     (pipeline, hop) groups, one 1 KiB block per wave-channel per step, whole
@@ -193,28 +195,35 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         total = (24 // (wpb + 1)) * 256 * wpb
     nslots = max_nslots
     slot_blocks = min(per8 * max(1, 8 // receivers), total // npos, TUNED_SLOT_BUDGET // 1024)
+    if op == _lib.OP_SENDRECV and npos == 2 and max_nslots == TUNED_NSLOTS and ll128:
+        # one hop under LL128, its origins on 20 of 32 CUs: four slots of
+        # 1.5 MiB in the room of three of 2.25 (-10 % against those; the Simple
+        # protocol takes a quarter longer that way and keeps the three)
+        slot_blocks, nslots = TUNED_SENDRECV_SLOT_BLOCKS, TUNED_SENDRECV_NSLOTS
     granule = wpb * (8 // math.gcd(real_pipes, 8))
     waves = max(granule, slot_blocks // pipes // granule * granule)
     return fit(pipes, nslots, waves, granule)
 
 
-def tuned_origin_cus(op: int, world: int, channels: int, waves_per_block: int) -> int:
-    """Of the 32 CUs of an XCD, how many the origins of a ring broadcast or
-    allgather get to themselves; ``channels`` = thread blocks per position of
-    the launch (the library ignores the number for small grids and other
-    collectives).  A CU keeps about 26 KB of loads in flight and a load from
-    HBM takes 2.5 us while the collective's stores saturate it, so the
-    origins' natural share of the CUs - one position in ``world`` - delivers
-    too little: measured best at 8 ranks is 9 of 32 (allgather of 8 x 128 MiB
-    3.38 -> 2.57 ms, broadcast of 64 MiB 0.237 -> 0.171 ms), 2.25 times the
-    natural share, which is what other ring lengths aim for.  The grid is
-    filled up to whole rounds over the CUs and has to stay resident (24
-    wavefronts per CU): the largest count up to the aim that fits."""
-    if op not in (_lib.OP_BROADCAST, _lib.OP_ALLGATHER) or world < 4 or channels % 8:
+def tuned_origin_cus(op: int, npos: int, channels: int, waves_per_block: int) -> int:
+    """Of the 32 CUs of an XCD, how many the origins of a sendrecv, a ring
+    broadcast or an allgather get to themselves; ``npos`` = positions of a
+    pipeline, ``channels`` = thread blocks per position of the launch (the
+    library ignores the number for small grids and other collectives).  A CU
+    keeps about 26 KB of loads in flight and a load from HBM takes 2.5 us
+    while the collective's stores saturate it, so the origins' natural share
+    of the CUs - one position in ``npos`` - delivers too little: measured
+    best at 8 positions is 9 of 32 (allgather of 8 x 128 MiB 3.38 -> 2.57 ms,
+    broadcast of 64 MiB 0.237 -> 0.171 ms), 2.25 times the natural share,
+    which is what other lengths aim for (a sendrecv over one hop: 20 of 32,
+    0.131 -> 0.119 ms for 256 MiB).  The grid is filled up to whole rounds
+    over the CUs and has to stay resident (24 wavefronts per CU): the largest
+    count up to the aim that fits."""
+    if op not in (_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_ALLGATHER) or npos < 2 or channels % 8:
         return 0
     groups, rounds_max = channels // 8, 24 // max(1, waves_per_block)
-    for n in range(max(1, min(16, round(72 / world))), 0, -1):
-        rounds = max(-(-groups // n), -(-(world - 1) * groups // (32 - n)))
+    for n in range(max(1, min(20, round(72 / npos))), 0, -1):
+        rounds = max(-(-groups // n), -(-(npos - 1) * groups // (32 - n)))
         if rounds <= rounds_max:
             return n
     return 0
@@ -427,7 +436,7 @@ class VirtualComm:
             raw = 960 if d.protocol == _lib.PROTO_LL128 else 1024
             d.slot_bytes, d.nslots, d.waves_per_channel_group = tuned_geometry(
                 op, self.world_size, route_len, threads, self.nslots, lds,
-                row_blocks=max(1, -(-row // raw)))
+                row_blocks=max(1, -(-row // raw)), ll128=d.protocol == _lib.PROTO_LL128)
         else:
             d.slot_bytes, d.nslots = self.slot_bytes, self.nslots
             step_blocks = self.slot_bytes // 1024 // pipes
@@ -457,8 +466,10 @@ class VirtualComm:
                 d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy
             elif self.origin_cus is not None:
                 d.origin_cus = self.origin_cus
-            elif self.auto_geometry:
-                d.origin_cus = tuned_origin_cus(op, self.world_size, channels, wpb)
+            elif self.auto_geometry and (op != _lib.OP_SENDRECV or d.protocol == _lib.PROTO_LL128):
+                d.origin_cus = tuned_origin_cus(
+                    op, max(route_len, 1) if op == _lib.OP_SENDRECV else self.world_size,
+                    channels, wpb)
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
         # test hooks travel beside the descriptor (mint_ring_launch_debug)

@@ -169,7 +169,7 @@ def test_compute_units_set_apart_for_origins_grow_the_grid():
     """origin_cus: the blocks of an XCD are taken in rounds of 32; in every
     round so many take an origin, the others the receiving positions; the grid
     is whole rounds.  Only large ring broadcasts / allgathers under the local
-    placement; ignored elsewhere."""
+    placement (and sendrecvs); ignored elsewhere."""
     L = _lib.lib()
     big = dict(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES, placement=1, cache_policy=2,
                slot_bytes=512 << 10, nslots=3, waves_per_channel_group=64)
@@ -181,14 +181,19 @@ def test_compute_units_set_apart_for_origins_grow_the_grid():
     bc = dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, cache_policy=2,
               slot_bytes=512 << 10, nslots=3, waves_per_channel_group=512)
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **bc)) == 8 * 32 * 5
-    # ignored: small grids, the spread placement, other collectives, short rings
+    # ignored: small grids, the spread placement, other collectives
     small = dict(big, waves_per_channel_group=16, slot_bytes=128 << 10)
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **small)) == 8 * 8 * 4
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **dict(big, placement=0, cache_policy=0))) == 8 * 8 * 16
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, placement=1, waves_per_channel_group=64)) == 8 * 9 * 16
-    two = make_op(origin_cus=9, world=2, **dict(big, slot_bytes=512 << 10, waves_per_channel_group=256))
-    two.ring[2] = 0
-    assert L.mint_ring_grid_blocks(two) == 2 * 2 * 64
+    # a sendrecv over one hop: 64 channels per XCD, 20 CUs for the origins (4 rounds), 12 for
+    # the destinations (6 rounds)
+    sr = make_op(origin_cus=20, op=_lib.OP_SENDRECV, dtype=_lib.BYTES, placement=1, cache_policy=2,
+                 route_len=2, slot_bytes=1536 << 10, nslots=4, waves_per_channel_group=1536)
+    sr.ring[0], sr.ring[1] = 0, 1
+    assert L.mint_ring_grid_blocks(sr) == 8 * 32 * 4
+    sr.threads_per_block = 128
+    assert L.mint_ring_grid_blocks(sr) == 8 * 32 * 8
 
 
 def test_plan_rejects_bad_buffers_and_rings():

@@ -46,14 +46,16 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     threads = common.TUNED_THREADS_REDUCING if pairs else 256
     slot, nslots, waves = common.tuned_geometry(op, world, 2, threads, common.TUNED_NSLOTS,
                                                 row_blocks=row_blocks)
-    assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and 1 <= nslots <= common.TUNED_NSLOTS
+    assert slot % 1024 == 0 and slot <= common.TUNED_SLOT_BUDGET and nslots >= 1
+    # (staging is allocated for TUNED_NSLOTS slots of TUNED_SLOT_BUDGET)
+    assert nslots * slot <= common.TUNED_NSLOTS * common.TUNED_SLOT_BUDGET
     multi = op == _lib.OP_ALLTOALL
     d = make_op(op=op, world=world, slot_bytes=slot, nslots=nslots, waves_per_channel_group=waves,
                 placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2, threads_per_block=threads,
                 dtype=_lib.F16 if reducing else _lib.BYTES)
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
-    d.origin_cus = common.tuned_origin_cus(op, world, pipes * -(-waves // (threads // 64)),
-                                           threads // 64)
+    d.origin_cus = common.tuned_origin_cus(op, 2 if op == _lib.OP_SENDRECV else world,
+                                           pipes * -(-waves // (threads // 64)), threads // 64)
     if op == _lib.OP_ALLTOALL:
         for r in range(8):
             d.output[r] = 0x40000000 + r * 0x1000000
@@ -81,6 +83,13 @@ def test_headline_geometry():
     assert common.tuned_geometry(_lib.OP_ALLREDUCE, 8, 0, 128, 3) == (512 * 1024, 3, 32)
     assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3) == (512 * 1024, 3, 64)
     assert common.tuned_geometry(_lib.OP_BROADCAST, 8, 0, 256, 3) == (512 * 1024, 3, 512)
+    assert common.tuned_geometry(_lib.OP_SENDRECV, 8, 2, 128, 3) == (1536 * 1024, 4, 1536)
+    assert common.tuned_geometry(_lib.OP_SENDRECV, 8, 3, 128, 3) == (1536 * 1024, 3, 1536)
+    assert common.tuned_geometry(_lib.OP_SENDRECV, 8, 2, 128, 3, ll128=False) == (2304 * 1024, 3, 2304)
+    assert common.tuned_origin_cus(_lib.OP_SENDRECV, 2, 768, 2) == 20
+    assert common.tuned_origin_cus(_lib.OP_ALLGATHER, 8, 8 * 16, 4) == 9
+    assert common.tuned_origin_cus(_lib.OP_BROADCAST, 8, 128, 4) == 9
+    assert common.tuned_origin_cus(_lib.OP_REDUCESCATTER, 8, 128, 4) == 0
     # a small message takes a small grid: the wave-channels are capped at the
     # blocks of one row, in whole thread blocks that the 8 XCDs divide
     assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=1) == (32 * 1024, 3, 4)
