@@ -9,12 +9,14 @@ ranks hold the same bits.
 
 Two ways to run it, same result bit for bit:
 
-* fused (default): one launch, one pass round the ring of 2 * world - 1
+* fused (``fused=True`` or ``MINTCCL_ALLREDUCE=fused``; the default below
+  32 MiB per rank): one launch, one pass round the ring of 2 * world - 1
   positions - what the reference plans.  Its two phases share the staging
   slots and the wavefronts.
-* split (``fused=False`` or ``MINTCCL_ALLREDUCE=split``): a reduce-scatter
-  launch followed by an allgather launch on the same chunks; each launch can
-  use the whole wavefront budget.
+* split (``fused=False`` or ``MINTCCL_ALLREDUCE=split``; the default from
+  32 MiB per rank): a reduce-scatter launch followed by an allgather launch on
+  the same chunks; each launch can use the whole wavefront budget, and the
+  allgather's origins get compute units of their own.
 """
 from __future__ import annotations
 
@@ -26,6 +28,13 @@ from . import _lib
 from ._ops import (check_buffer, comm_or_default, nbytes, reduce_dtype, ring_of,
                    same_everywhere)
 from .common import VirtualComm
+
+
+# From this size per rank on, two launches are faster than one pass (measured
+# on MI355X, 8 ranks, f16: 104 / 110 us at 16 MiB, 199 / 192 at 32 MiB, 1510 /
+# 1384 at 256 MiB; below, the second launch costs more than it gains: 12 / 18 us
+# at 64 KiB).
+SPLIT_FROM_BYTES = 32 << 20
 
 
 def chunk_bytes(count: int, world: int) -> int:
@@ -46,7 +55,8 @@ def allreduce(buff: torch.Tensor, comm: VirtualComm | None = None,
     dtype = same_everywhere(posted, "dtype", "the dtype")
     ptrs = {r: info["ptr"] for r, info in posted.items()}
     if fused is None:
-        fused = os.getenv("MINTCCL_ALLREDUCE", "fused").lower() != "split"
+        choice = os.getenv("MINTCCL_ALLREDUCE", "").lower()
+        fused = choice != "split" if choice else count < SPLIT_FROM_BYTES
     ring = ring_of(comm)
     if fused:
         comm.launch(comm.make_op(_lib.OP_ALLREDUCE, dtype, count, ptrs, ptrs, ring))
