@@ -110,9 +110,9 @@ class Timer:
 
 
 # Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
-# step.  Alltoall: 2 slots of 640 KiB per 8 receiving ranks, 5760 wavefronts in
-# all (from about 6100 on the grid no longer runs as one wave of blocks and the
-# time jumps by a third).  Everything else: 3 slots of 512 KiB, 4608
+# step.  Alltoall: 6 slots, 2560 wavefronts in all (Simple protocol: 2 slots,
+# 5760 wavefronts).  Everything else: 3 slots
+# of 512 KiB, 4608
 # wavefronts (reducescatter: 3 slots of 448 KiB, 56 wave-channels per
 # (row, hop) instead of 64: 1.5 - 2 % faster; broadcast and allgather with CUs
 # set apart for their origins, tuned_origin_cus);
@@ -126,9 +126,10 @@ TUNED_TOTAL_WAVES = 4608
 TUNED_SLOT_BLOCKS = 512
 TUNED_SLOT_BLOCKS_REDUCESCATTER = 448
 TUNED_NSLOTS = 3
-TUNED_TOTAL_WAVES_MULTI = 5760
-TUNED_SLOT_BLOCKS_MULTI = 640
-TUNED_NSLOTS_MULTI = 2
+TUNED_TOTAL_WAVES_ALLTOALL = 2560
+TUNED_NSLOTS_ALLTOALL = 6
+TUNED_TOTAL_WAVES_ALLTOALL_SIMPLE = 5760
+TUNED_NSLOTS_ALLTOALL_SIMPLE = 2
 TUNED_SLOT_BUDGET = 2304 * 1024
 TUNED_THREADS_REDUCING = 128
 TUNED_SENDRECV_SLOT_BLOCKS = 1536
@@ -163,11 +164,19 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
 
     if op == _lib.OP_ALLTOALL:
         # world x world pipelines of two positions; a rank's slot has one share
-        # per source rank
-        total = TUNED_TOTAL_WAVES_MULTI
+        # per source rank.  Few wave-channels and many small slots, origins on
+        # 20 of 32 CUs: 8 x 256 MiB 1.13 -> 0.91 ms (LL128) against 2 slots and
+        # 5760 wavefronts with origins and destinations on half of the CUs each.
+        # The Simple protocol takes twice as long that way and keeps 2 slots
+        # and 5760 wavefronts.
+        total = TUNED_TOTAL_WAVES_ALLTOALL if ll128 else TUNED_TOTAL_WAVES_ALLTOALL_SIMPLE
         granule = wpb * (8 // math.gcd(world * world, 8))      # whole channels for every XCD
         waves = max(granule, total // (2 * world * world) // granule * granule)
-        return fit(world, min(max_nslots, TUNED_NSLOTS_MULTI), waves, granule)
+        if not ll128:
+            nslots = min(max_nslots, TUNED_NSLOTS_ALLTOALL_SIMPLE)
+        else:
+            nslots = TUNED_NSLOTS_ALLTOALL if max_nslots == TUNED_NSLOTS else max_nslots
+        return fit(world, nslots, waves, granule)
     if op in (_lib.OP_TREE_BROADCAST, _lib.OP_TREE_REDUCE):
         # one wavefront per (node, wave-channel); a reducing node's slot has a
         # share per child
@@ -207,7 +216,7 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
 
 def tuned_origin_cus(op: int, npos: int, channels: int, waves_per_block: int) -> int:
     """Of the 32 CUs of an XCD, how many the origins of a sendrecv, a ring
-    broadcast or an allgather get to themselves; ``npos`` = positions of a
+    broadcast, an allgather or an alltoall get to themselves; ``npos`` = positions of a
     pipeline, ``channels`` = thread blocks per position of the launch (the
     library ignores the number for small grids and other collectives).  A CU
     keeps about 26 KB of loads in flight and a load from HBM takes 2.5 us
@@ -216,10 +225,11 @@ def tuned_origin_cus(op: int, npos: int, channels: int, waves_per_block: int) ->
     best at 8 positions is 9 of 32 (allgather of 8 x 128 MiB 3.38 -> 2.57 ms,
     broadcast of 64 MiB 0.237 -> 0.171 ms), 2.25 times the natural share,
     which is what other lengths aim for (a sendrecv over one hop: 20 of 32,
-    0.131 -> 0.119 ms for 256 MiB).  The grid is filled up to whole rounds
+    0.131 -> 0.119 ms for 256 MiB; alltoall, whose pipelines are single hops:
+    the same 20).  The grid is filled up to whole rounds
     over the CUs and has to stay resident (24 wavefronts per CU): the largest
     count up to the aim that fits."""
-    if op not in (_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_ALLGATHER) or npos < 2 or channels % 8:
+    if op not in (_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_ALLGATHER, _lib.OP_ALLTOALL) or npos < 2 or channels % 8:
         return 0
     groups, rounds_max = channels // 8, 24 // max(1, waves_per_block)
     for n in range(max(1, min(20, round(72 / npos))), 0, -1):
@@ -466,10 +476,11 @@ class VirtualComm:
                 d.cache_policy = 0 if self.cache_policy == 2 else self.cache_policy
             elif self.origin_cus is not None:
                 d.origin_cus = self.origin_cus
-            elif self.auto_geometry and (op != _lib.OP_SENDRECV or d.protocol == _lib.PROTO_LL128):
-                d.origin_cus = tuned_origin_cus(
-                    op, max(route_len, 1) if op == _lib.OP_SENDRECV else self.world_size,
-                    channels, wpb)
+            elif self.auto_geometry and (op not in (_lib.OP_SENDRECV, _lib.OP_ALLTOALL)
+                                         or d.protocol == _lib.PROTO_LL128):
+                npos = {_lib.OP_SENDRECV: max(route_len, 1), _lib.OP_ALLTOALL: 2}.get(
+                    op, self.world_size)
+                d.origin_cus = tuned_origin_cus(op, npos, channels, wpb)
         d.spin_budget = self.spin_budget
         d.status = self.status.data_ptr()
         # test hooks travel beside the descriptor (mint_ring_launch_debug)

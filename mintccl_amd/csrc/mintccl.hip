@@ -263,7 +263,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     // the XCD-local mapping deals whole channels to XCDs
     if (op->placement == MINT_PLACE_LOCAL && (a.pipes * a.blocks_per_group) % kXcds)
         return MINT_ERR_GEOMETRY;
-    // Large sendrecvs, ring broadcasts and allgathers under the local placement: origins
+    // Large sendrecvs, ring broadcasts, allgathers and alltoalls under the local placement: origins
     // on CUs which they have to themselves, as many as the caller names
     // (take_seat); the grid grows by the blocks that find nothing to do.
     a.origin_cus = 0;
@@ -274,7 +274,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         plan->blocks_plain = plan->blocks;
         if (op->placement == MINT_PLACE_LOCAL && origin_cus > 0 && npos >= 2 && groups >= 8 &&
             (op->op == MINT_OP_BROADCAST || op->op == MINT_OP_ALLGATHER ||
-             op->op == MINT_OP_SENDRECV)) {
+             op->op == MINT_OP_SENDRECV || op->op == MINT_OP_ALLTOALL)) {
             const int others = kCusPerXcd - origin_cus;
             const int r0 = (groups + origin_cus - 1) / origin_cus;
             const int r1 = ((npos - 1) * groups + others - 1) / others;

@@ -54,7 +54,9 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
                 placement=_lib.PLACE_LOCAL, cache_policy=2, route_len=2, threads_per_block=threads,
                 dtype=_lib.F16 if reducing else _lib.BYTES)
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
-    d.origin_cus = common.tuned_origin_cus(op, 2 if op == _lib.OP_SENDRECV else world,
+    if op == _lib.OP_ALLTOALL:
+        pipes = world * world
+    d.origin_cus = common.tuned_origin_cus(op, 2 if op in (_lib.OP_SENDRECV, _lib.OP_ALLTOALL) else world,
                                            pipes * -(-waves // (threads // 64)), threads // 64)
     if op == _lib.OP_ALLTOALL:
         for r in range(8):
@@ -71,7 +73,7 @@ def test_tuned_geometry_is_always_launchable(op, world, row_blocks):
     assert blocks % 8 == 0
     # (CUs set apart for origins fill the grid up to whole rounds over the 256
     # CUs, at most 24 wavefronts each)
-    budget = common.TUNED_TOTAL_WAVES_MULTI if multi else common.TUNED_TOTAL_WAVES
+    budget = common.TUNED_TOTAL_WAVES_ALLTOALL_SIMPLE if multi else common.TUNED_TOTAL_WAVES
     assert blocks * (threads // 64) <= (24 * 256 if d.origin_cus else budget)
     d.origin_cus = 0
     assert 0 < _lib.lib().mint_ring_grid_blocks(d) <= blocks
@@ -90,6 +92,9 @@ def test_headline_geometry():
     assert common.tuned_origin_cus(_lib.OP_ALLGATHER, 8, 8 * 16, 4) == 9
     assert common.tuned_origin_cus(_lib.OP_BROADCAST, 8, 128, 4) == 9
     assert common.tuned_origin_cus(_lib.OP_REDUCESCATTER, 8, 128, 4) == 0
+    assert common.tuned_geometry(_lib.OP_ALLTOALL, 8, 0, 128, 3) == (8 * 20 * 1024, 6, 20)
+    assert common.tuned_geometry(_lib.OP_ALLTOALL, 8, 0, 128, 3, ll128=False) == (8 * 44 * 1024, 2, 44)
+    assert common.tuned_origin_cus(_lib.OP_ALLTOALL, 2, 64 * 10, 2) == 20
     # a small message takes a small grid: the wave-channels are capped at the
     # blocks of one row, in whole thread blocks that the 8 XCDs divide
     assert common.tuned_geometry(_lib.OP_ALLGATHER, 8, 0, 256, 3, row_blocks=1) == (32 * 1024, 3, 4)
