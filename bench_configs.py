@@ -6,6 +6,8 @@ adder folded in ring order).
 
     python bench_configs.py [--quick]
 
+  config 1  LL128 line codec alone: pack + unpack of 1 MiB (524,288 fp16) and of 256 MiB,
+            the reference's 8-lane pair layout and the 64-lane block layout
   config 2  sendrecv 256 MiB fp16, rank 0 -> rank 1: LL128, Simple, direct copy
   config 3  ring broadcast 64 MiB, 8 ranks, 8 x 512 KiB slots
   config 4  ring reduce and reducescatter, 32 Mi elements per rank, f16 / bf16 / f32
@@ -36,7 +38,7 @@ sys.path.insert(0, ROOT)
 
 import torch  # noqa: E402
 
-from mintccl_amd import _lib, primitive, sendrecv_buffer, sendrecv_direct  # noqa: E402
+from mintccl_amd import _lib, primitive, protocol, sendrecv_buffer, sendrecv_direct  # noqa: E402
 from mintccl_amd.allgather import allgather  # noqa: E402
 from mintccl_amd.broadcast import broadcast  # noqa: E402
 from mintccl_amd.common import VirtualComm  # noqa: E402
@@ -92,6 +94,29 @@ def comm_for(world: int, proto: int, slots=None, **kw) -> VirtualComm:
     if slots is not None:
         kw.update(buff_size_=slots[0] * slots[1], nslots=slots[0])
     return VirtualComm(world_size=world, device=DEV, protocol=proto, **kw)
+
+
+def config1(reps: int) -> None:
+    """The codec on its own: raw -> lines -> raw (mint_ll128_pack / _unpack),
+    flag = line number from 1 as in the reference.  Bytes that cross HBM:
+    raw read + lines written, lines read + raw written."""
+    for n in (524288, 134217728):
+        g = torch.Generator(device=DEV).manual_seed(0)
+        raw = torch.empty(n, device=DEV, dtype=torch.float16).uniform_(-1, 1, generator=g)
+        back = torch.empty_like(raw)
+        bad = torch.zeros(1, dtype=torch.int64, device=DEV)
+        for name, layout in (("pair (8 lanes, the reference's)", protocol.LAYOUT_PAIR),
+                             ("wave64 (1 KiB blocks)", protocol.LAYOUT_WAVE64)):
+            msg = torch.empty(protocol.packed_bytes(n * 2, layout), dtype=torch.uint8, device=DEV)
+
+            def step():
+                protocol.pack(raw, 1, layout, out=msg)
+                protocol.unpack(msg, back, 1, layout, bad_flags=bad)
+            ms = time_ms(step, reps * (20 if n < 1 << 20 else 1))
+            ok = bool(torch.equal(raw, back)) and int(bad.item()) == 0
+            emit(config=1, op="pack + unpack", layout=name, bytes=n * 2, us=round(ms * 1e3, 2),
+                 ok=ok, hbm_bytes=2 * (n * 2 + msg.numel()))
+        del raw, back, msg
 
 
 def config2(reps: int) -> None:
@@ -423,7 +448,7 @@ def main() -> int:
     ap.add_argument("--staging", choices=("both", "reference", "tuned"), default="both")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
     ap.add_argument("--only", type=int, default=0,
-                    help="run one config (2..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring)")
+                    help="run one config (1..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring)")
     ap.add_argument("--shard-log2", default="",
                     help="config 5: only these shard sizes (log2 of bytes, comma separated)")
     ap.add_argument("--tree-log2", default="10,14,17,20,23,26",
@@ -433,6 +458,8 @@ def main() -> int:
     STAGING = ("reference", "tuned") if args.staging == "both" else (args.staging,)
     reps = 3 if args.quick else 8
     torch.cuda.set_device(DEV)
+    if args.only in (0, 1):
+        config1(reps)
     if args.only in (0, 2):
         config2(reps)
     if args.only in (0, 3):
