@@ -634,6 +634,50 @@ def test_a_lost_producer_times_out_instead_of_hanging(dev):
         assert torch.equal(b.cpu(), host[2])
 
 
+@pytest.mark.parametrize("op", ["broadcast", "allgather", "sendrecv"])
+def test_a_spin_limit_of_one_ends_every_wait(dev, op):
+    """Large launches at the tuned geometry (origins on compute units of their
+    own, fetching ahead, their credit read through the scalar unit) with a
+    spin limit of one poll: whoever has to wait gives up at once, every
+    wavefront ends, the launch reports a timeout - and the same memory works
+    again afterwards."""
+    from mintccl_amd import _lib
+    from mintccl_amd.common import RingTimeout
+    world, n = 8, 4 << 20
+    g = torch.Generator().manual_seed(7)
+    host = [torch.randint(0, 256, (world, n), dtype=torch.uint8, generator=g) for _ in range(world)]
+    bufs = [h.to(dev) for h in host]
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    ring_order = list(range(world)) + [0]
+
+    def describe(comm):
+        if op == "broadcast":
+            return comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, world * n, {0: ptrs[0]},
+                                {r: p for r, p in ptrs.items() if r}, ring_order, root=0)
+        if op == "allgather":
+            return comm.make_op(_lib.OP_ALLGATHER, _lib.BYTES, n, ptrs, ptrs, ring_order, row_stride=n)
+        return comm.make_op(_lib.OP_SENDRECV, _lib.BYTES, world * n, {0: ptrs[0]}, {1: ptrs[1]},
+                            [0, 1], route_len=2)
+    comm = make_comm(world, spin_budget=1)
+    d = describe(comm)
+    assert d.origin_cus > 0
+    comm.launch(d)
+    with pytest.raises(RingTimeout):
+        comm.check()
+    comm.spin_budget = 400000
+    for r in range(world):
+        bufs[r].copy_(host[r])
+    comm.launch(describe(comm))
+    comm.check()
+    if op == "broadcast":
+        assert all(torch.equal(b.cpu(), host[0]) for b in bufs)
+    elif op == "allgather":
+        want = torch.stack([host[r][r] for r in range(world)])
+        assert all(torch.equal(b.cpu(), want) for b in bufs)
+    else:
+        assert torch.equal(bufs[1].cpu(), host[0])
+
+
 def test_residency_is_checked(dev):
     from mintccl_amd import _lib
     world = 8
