@@ -957,11 +957,9 @@ __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib) {
         // sit on CUs of their own and the polls of the others, answered by
         // the L2, never queue behind a load from HBM in a CU's memory
         // pipeline.  The ring walks are fastest that way (an allgather whose
-        // CUs hold a mix of positions takes 4 - 10 % longer).  The tree and
-        // the temporal allgather, where the loading position of a wave-channel
-        // is one of few or changes from phase to phase, gain 6 - 10 % from a
-        // mix: seat_turn turns the positions by two after every round over the
-        // CUs.
+        // CUs hold a mix of positions takes 4 - 10 % longer).  The tree gains
+        // 10 % from a mix: seat_turn turns the positions by two after every
+        // round over the CUs.
         int q = y / npos;
         st.h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
         if (a.origin_cus) {
