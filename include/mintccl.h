@@ -181,7 +181,7 @@ typedef struct {
     uint32_t origin_cus;   /* 0, or of the 32 compute units of an XCD so many
                               hold nothing but origins (the positions that
                               read the caller's rows from HBM): SENDRECV,
-                              BROADCAST, ALLGATHER(_TEMPORAL) and ALLTOALL under MINT_PLACE_LOCAL
+                              BROADCAST, TREE_BROADCAST, ALLGATHER(_TEMPORAL) and ALLTOALL under MINT_PLACE_LOCAL
                               with at least 64 thread blocks per position,
                               below 32; ignored elsewhere, and
                               where the larger grid it needs (blocks with

@@ -230,7 +230,7 @@ def tuned_origin_cus(op: int, npos: int, channels: int, waves_per_block: int) ->
     over the CUs and has to stay resident (24 wavefronts per CU): the largest
     count up to the aim that fits."""
     if op not in (_lib.OP_SENDRECV, _lib.OP_BROADCAST, _lib.OP_ALLGATHER, _lib.OP_ALLTOALL,
-                  _lib.OP_ALLGATHER_TEMPORAL) or npos < 2 or channels % 8:
+                  _lib.OP_ALLGATHER_TEMPORAL, _lib.OP_TREE_BROADCAST) or npos < 2 or channels % 8:
         return 0
     groups, rounds_max = channels // 8, 24 // max(1, waves_per_block)
     for n in range(max(1, min(20, round(72 / npos))), 0, -1):

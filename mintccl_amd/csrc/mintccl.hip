@@ -274,7 +274,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         plan->blocks_plain = plan->blocks;
         if (op->placement == MINT_PLACE_LOCAL && origin_cus > 0 && npos >= 2 && groups >= 8 &&
             (op->op == MINT_OP_BROADCAST || op->op == MINT_OP_ALLGATHER ||
-             op->op == MINT_OP_SENDRECV || op->op == MINT_OP_ALLTOALL || temporal)) {
+             op->op == MINT_OP_SENDRECV || op->op == MINT_OP_ALLTOALL || temporal ||
+             op->op == MINT_OP_TREE_BROADCAST)) {
             const int others = kCusPerXcd - origin_cus;
             const int r0 = (groups + origin_cus - 1) / origin_cus;
             const int r1 = ((npos - 1) * groups + others - 1) / others;

@@ -100,8 +100,85 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
     u32x4 ahead = {0u, 0u, 0u, 0u};
     if (load && (uint32_t)w < nfull) ahead = ll_fetch_raw(in_row, row_bytes, (uint32_t)w, true, m);
 
-    uint32_t slot = 0;
-    for (uint32_t s = 0; s < a.steps; ++s) {
+    uint32_t slot = 0, s = 0;
+    if (!reduce && h == 0 && STCP == CP_NONE && K == 1u && nout > 0) {
+        // The root of a broadcast, one block per step, XCD-local staging, on
+        // compute units set apart for it (origin_cus): rows fetched kAhead
+        // steps ahead, the children's credit words read through the scalar
+        // unit so that looking at them does not wait for the fetches (a load
+        // from HBM takes 2.5 us under the tree's stores).  Whole blocks only;
+        // the ragged end of the buffer takes the loop below.
+        constexpr uint32_t kAhead = 4;
+        const uint32_t whole = nfull > (uint32_t)w ? (nfull - 1u - (uint32_t)w) / a.step_blocks + 1u : 0u;
+        const uint32_t deep = whole < a.steps ? whole : a.steps;
+        if (deep) {
+            u32x4 vv[kAhead];
+            auto fetch = [&](uint32_t of_step) __attribute__((always_inline)) {
+                uint32_t g = of_step * a.step_blocks + (uint32_t)w;
+                g = g < nfull ? g : nfull - 1u;              // beyond the whole blocks: any valid address
+                return ll_fetch_raw(in_row, row_bytes, g, true, m);
+            };
+            // (the prologue issues the queue a later step finds: stores stand in
+            // for a step's two sends, to an unused part of a credit line)
+            uint64_t* const pad = const_cast<uint64_t*>(out_tail[0]) + 8;
+            vv[0] = fetch(0u);
+#pragma unroll
+            for (uint32_t d = 1; d < kAhead; ++d) {
+                compiler_fence();
+                st64_local(pad, 0ull);
+                st64_local(pad, 0ull);
+                compiler_fence();
+                vv[d] = fetch(d);
+            }
+            auto step = [&](auto phase) __attribute__((always_inline)) {
+                constexpr int B = decltype(phase)::value;
+                const uint32_t tag = (epoch << 20) | (s + 1u);
+                const uint32_t need = s >= a.nslots ? s - a.nslots + 1 : 0;
+#pragma unroll
+                for (int j = 0; j < kTreeArity; ++j) {
+                    if (j >= nout) continue;
+                    for (uint32_t spins = 0; credits_seen[j] < need; ++spins) {
+                        const uint64_t cw = ld64_scalar(out_tail[j]);
+                        if ((uint32_t)(cw >> 32) == epoch && (uint32_t)cw >= need) {
+                            credits_seen[j] = (uint32_t)cw;
+                            break;
+                        }
+                        if (spins >= a.spin_budget ||
+                            ((spins & 63u) == 63u &&
+                             __builtin_amdgcn_readfirstlane(ld32_agent_apart(a.status + 3)) != 0u)) {
+                            report_timeout(a.status, 0, h, w, s);
+                            __builtin_amdgcn_endpgm();
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                }
+                const uint32_t at = slot * a.slot_bytes + (uint32_t)w * kBlockMsg;
+                const u32x4 x = ll_arrange(vv[B], true, m);
+                // (a root with one child sends the block twice to the same place)
+                ll_send<STCP>(out0, at, x, tag, m);
+                ll_send<STCP>(nout > 1 ? out1 : out0, at, x, tag, m);
+                compiler_fence();
+                vv[B] = fetch(s + kAhead);
+                slot = slot + 1 == a.nslots ? 0 : slot + 1;
+                ++s;
+            };
+            while (s < deep) {
+                step(std::integral_constant<int, 0>{});
+                if (s >= deep) break;
+                step(std::integral_constant<int, 1>{});
+                if (s >= deep) break;
+                step(std::integral_constant<int, 2>{});
+                if (s >= deep) break;
+                step(std::integral_constant<int, 3>{});
+            }
+            // the loop below fetches its own rows one block ahead
+            if (s < a.steps) {
+                const uint32_t g = s * a.step_blocks + (uint32_t)w;
+                if (g < nfull) ahead = ll_fetch_raw(in_row, row_bytes, g, true, m);
+            }
+        }
+    }
+    for (; s < a.steps; ++s) {
         const uint32_t tag = (epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the receiver has emptied the slot
         // this step goes into
