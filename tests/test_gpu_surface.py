@@ -242,6 +242,67 @@ def test_self_tests_over_world_sizes_and_knobs(monkeypatch, capsys, world, knobs
 
 
 @pytest.mark.gpu
+def test_captured_large_collectives_replay(dev):
+    """The same for messages large enough for the tuned launches with compute
+    units set apart for the origins (allgather in both schedules, broadcast,
+    sendrecv over one hop, alltoall): three replays against eager runs."""
+    from mintccl_amd import sendrecv_buffer
+    from mintccl_amd.allgather import allgather
+    from mintccl_amd.alltoall import alltoall
+    from mintccl_amd.broadcast import broadcast
+    world, n = 8, (1 << 20) + 40
+    comm = make_comm(world, device_epoch=True)
+    eager = make_comm(world)
+    ins = [torch.zeros(world, n, dtype=torch.float16, device=dev) for _ in range(world)]
+
+    def buffers():
+        return ([torch.zeros_like(x) for x in ins], [torch.zeros_like(x) for x in ins],
+                [torch.zeros(world * n, dtype=torch.float16, device=dev) for _ in range(world)],
+                [torch.zeros_like(x) for x in ins], [torch.zeros_like(x) for x in ins])
+
+    def sequence(cm, a, t, c, x, y):
+        for r in range(world):
+            a[r].copy_(ins[r]); t[r].copy_(ins[r]); c[r].copy_(ins[r].view(-1)); x[r].copy_(ins[r])
+        cm.run(lambda r: allgather(a[r], cm))
+        cm.run(lambda r: allgather(t[r], cm, schedule="temporal"))
+        cm.run(lambda r: broadcast(c[r], 5, cm))
+        cm.run(lambda r: alltoall(x[r], y[r], cm))
+        with cm.rank(2):
+            sendrecv_buffer.send(a[2], 6, cm)     # the gathered rows land in rank 6's alltoall input
+        with cm.rank(6):
+            sendrecv_buffer.recv(x[6], 2, cm)
+        cm.run(lambda r: sendrecv_buffer.sync(cm))
+
+    def fill(seed):
+        for r, h in enumerate(rank_rows(world, n, "f16", seed0=seed)):
+            ins[r].copy_(h.to(dev))
+
+    fill(300)
+    got, want = buffers(), buffers()
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        sequence(comm, *got)                      # warm up outside the capture
+    side.synchronize()
+    comm.check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sequence(comm, *got)
+    for replay in range(3):
+        fill(400 + 10 * replay)
+        sequence(eager, *want)
+        eager.check()
+        graph.replay()
+        torch.cuda.synchronize()
+        comm.check()
+        for g, w in zip(got, want):
+            for r in range(world):
+                assert torch.equal(g[r], w[r]), replay
+    # sanity of what was compared: the allgathers gathered, the broadcast spread rank 5's buffer
+    assert all(torch.equal(want[0][r][q], ins[q][q]) for r in range(world) for q in range(world))
+    assert all(torch.equal(want[1][r], want[0][r]) for r in range(world))
+    assert torch.equal(want[3][6], want[0][2]) and torch.equal(want[3][5], ins[5])
+
+
 def test_captured_collectives_replay(dev):
     """A captured sequence of collectives (epoch in device memory) is replayed
     several times, with eager work and fresh inputs in between; every replay
