@@ -453,6 +453,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // flight: it has a whole group's time to come back from HBM.  The other
     // groups (the ragged end of a row, a step that is only partly filled) take
     // the guarded body and load their own rows on the spot.
+    // Simple protocol, copying positions that send: sends before saves / fetch
+    // (an origin, or a position that also keeps a copy: the operations that
+    // follow the sends are then the same number on every path)
+    constexpr bool kSendsFirst = PROTO == PROTO_SIMPLE && DT == DT_BYTES && RoleT::send && !LDSF &&
+                                 (RoleT::save || !RoleT::recv);
     auto run_group = [&](auto whole_tag, auto parity_tag) MINT_INLINE_LAMBDA -> bool {
         constexpr bool WHOLE = decltype(whole_tag)::value;
         constexpr int P = decltype(parity_tag)::value;
@@ -493,6 +498,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     return false;
                 }
                 if (timing) t_lds += wall_clock64() - t0;
+            } else if (WHOLE && kSendsFirst && !role.recv) {
+                // (a Simple origin fetches ahead after its sends, see below)
             } else if (WHOLE) {
                 fetch_ahead(qn, vnext);
             } else {
@@ -558,6 +565,13 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     x = r[u];
                 }
             }
+            if (WHOLE && kSendsFirst) {
+                // the sends of the whole group first: the counter that follows
+                // them then waits for them only
+                st128<STCP>(nxt, q.msg_off(geom, share_send, u) + m.lane * 16u, x);
+                v[u] = x;
+                continue;
+            }
             if (role.save) {
                 if (PROTO == PROTO_LL128) {
                     ll_save_raw(out_row, row_bytes, q.g[u], full, m, x);
@@ -574,6 +588,17 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     st128<STCP>(nxt, q.msg_off(geom, share_send, u) + m.lane * 16u, x);
             }
         }
+        if (WHOLE && kSendsFirst) {
+            compiler_fence();
+            if (role.save) {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    st128_row(out_row + (uint64_t)q.g[u] * kBlockRawSimple + m.lane * 16u, v[u]);
+            } else if (!LDSF) {
+                fetch_ahead(qn, vnext);
+            }
+            compiler_fence();
+        }
         if (q.last) {
             // Simple protocol: this wave-channel has taken every line of step s
             // out of its slot (the stores above carry what the loads returned).
@@ -584,7 +609,13 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             if (PROTO == PROTO_SIMPLE && role.send) {
                 // Simple protocol: data first, then the step counter.  The data
                 // loads of the receiver skip the L1 (LDCP), so no invalidate.
-                wait_stores_visible();
+                // Where the group's sends went out first, the U operations
+                // issued after them - a receiver's saves to HBM, an origin's
+                // fetch ahead - and the credit post may stay in flight.
+                if (WHOLE && kSendsFirst)
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(U + (RoleT::recv ? 1 : 0)) : "memory");
+                else
+                    wait_stores_visible();
                 if (lane_id() == 0) {
                     if (STCP == CP_NONE) st64_local(nxt_head, flag_hi | (uint64_t)(s + 1));
                     else st64_agent(nxt_head, flag_hi | (uint64_t)(s + 1));
