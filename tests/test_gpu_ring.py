@@ -634,6 +634,54 @@ def test_a_lost_producer_times_out_instead_of_hanging(dev):
         assert torch.equal(b.cpu(), host[2])
 
 
+@pytest.mark.parametrize("world", [2, 3, 5, 6, 7])
+def test_large_copying_collectives_over_world_sizes(dev, world):
+    """Messages large enough for the full tuned grids, where the origins get
+    compute units of their own (a different count for every ring length),
+    at odd row sizes: allgather in both schedules, ring and tree broadcast,
+    alltoall, sendrecv over one hop."""
+    from mintccl_amd import _lib
+    n = (3 << 20) + 5 * world + 1                    # bytes per row
+    g = torch.Generator().manual_seed(world)
+    host = [torch.randint(0, 256, (world, n), dtype=torch.uint8, generator=g) for _ in range(world)]
+    ring_order = list(range(world)) + [0]
+    comm = make_comm(world)
+    want = torch.stack([host[r][r] for r in range(world)])
+    for op in (_lib.OP_ALLGATHER, _lib.OP_ALLGATHER_TEMPORAL):
+        bufs = [h.to(dev) for h in host]
+        ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+        d = comm.make_op(op, _lib.BYTES, n, ptrs, ptrs, ring_order, row_stride=n)
+        assert d.origin_cus > 0
+        comm.launch(d)
+        comm.check()
+        assert all(torch.equal(b.cpu(), want) for b in bufs)
+    root = world - 1
+    for op in (_lib.OP_BROADCAST, _lib.OP_TREE_BROADCAST):
+        bufs = [h.to(dev) for h in host]
+        ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+        d = comm.make_op(op, _lib.BYTES, world * n, {root: ptrs[root]},
+                         {r: p for r, p in ptrs.items() if r != root}, ring_order, root=root)
+        assert d.origin_cus > 0
+        comm.launch(d)
+        comm.check()
+        assert all(torch.equal(b.cpu(), host[root]) for b in bufs)
+    bufs = [h.to(dev) for h in host]
+    outs = [torch.zeros_like(b) for b in bufs]
+    d = comm.make_op(_lib.OP_ALLTOALL, _lib.BYTES, n, {r: bufs[r].data_ptr() for r in range(world)},
+                     {r: outs[r].data_ptr() for r in range(world)}, ring_order, row_stride=n)
+    assert d.origin_cus > 0
+    comm.launch(d)
+    comm.check()
+    for r in range(world):
+        assert torch.equal(outs[r].cpu(), torch.stack([host[q][r] for q in range(world)]))
+    d = comm.make_op(_lib.OP_SENDRECV, _lib.BYTES, world * n, {0: bufs[0].data_ptr()},
+                     {world - 1: outs[world - 1].data_ptr()}, [0, world - 1], route_len=2)
+    assert d.origin_cus > 0
+    comm.launch(d)
+    comm.check()
+    assert torch.equal(outs[world - 1].cpu(), host[0])
+
+
 @pytest.mark.parametrize("op", ["broadcast", "allgather", "sendrecv"])
 def test_a_spin_limit_of_one_ends_every_wait(dev, op):
     """Large launches at the tuned geometry (origins on compute units of their
