@@ -682,6 +682,27 @@ def test_large_copying_collectives_over_world_sizes(dev, world):
     assert torch.equal(outs[world - 1].cpu(), host[0])
 
 
+def test_origin_cus_that_would_not_be_resident_fall_back_to_the_plain_order(dev):
+    """16 of 32 CUs for the origins of an 8-rank allgather with 80 wave-channels
+    per (row, hop) would take 9 rounds over the CUs, more than are resident:
+    the launch runs in the plain order instead of failing."""
+    from mintccl_amd import _lib
+    world, n = 8, (2 << 20) + 16
+    comm = make_comm(world, buff_size_=2 * 640 * 1024, nslots=2, waves_per_rank=640,
+                     placement=1, cache_policy=2, origin_cus=16)
+    g = torch.Generator().manual_seed(3)
+    host = [torch.randint(0, 256, (world, n), dtype=torch.uint8, generator=g) for _ in range(world)]
+    bufs = [h.to(dev) for h in host]
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    d = comm.make_op(_lib.OP_ALLGATHER, _lib.BYTES, n, ptrs, ptrs, list(range(world)) + [0], row_stride=n)
+    d.flag_epoch = 1                              # (the launch sets its own)
+    assert d.origin_cus == 16 and _lib.lib().mint_ring_grid_blocks(d) == 8 * 32 * 9
+    comm.launch(d)
+    comm.check()
+    want = torch.stack([host[r][r] for r in range(world)])
+    assert all(torch.equal(b.cpu(), want) for b in bufs)
+
+
 @pytest.mark.parametrize("op", ["broadcast", "allgather", "sendrecv"])
 def test_a_spin_limit_of_one_ends_every_wait(dev, op):
     """Large launches at the tuned geometry (origins on compute units of their
