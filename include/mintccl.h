@@ -193,6 +193,7 @@ typedef struct {
     uint32_t reserved1;    /* 0 */
 } mint_ring_op;
 
+/* 100 * major + minor of the descriptor layout: 101 = mint_ring_op with origin_cus. */
 int mint_version(void);
 const char* mint_strerror(int err);
 

@@ -23,7 +23,7 @@ static __device__ __align__(256) unsigned char scratch[MINT_STATIC_SCRATCH_BYTES
 
 namespace {
 
-constexpr int kVersion = 100;   // 0.1.0
+constexpr int kVersion = 101;   // 0.1.1: mint_ring_op grew by origin_cus
 constexpr uint32_t kDefaultSpinBudget = 4000000u;
 constexpr uint32_t kMaxEpoch = 4095u;          // 12 bits of every sector tag
 constexpr uint32_t kMaxSteps = (1u << 20) - 1; // 20 bits of every sector tag
