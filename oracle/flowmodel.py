@@ -28,6 +28,10 @@ start of a round, before the slot has been drained - ``3_sendrecv_buffer.py:49-5
 with ``protocol.py:183-189``); ``drop=(h, s, l)`` loses one line write.  Both
 must be caught, which is how the tests know the checker has teeth.
 
+``explore_temporal`` does the same for the temporal allgather, where one agent
+per position serves a different rank in every phase and the ranks' credit
+words change hands (``mintccl_amd/csrc/temporal.hpp``).
+
 Pinning: this is a model of the build's own protocol, checked by invariants
 (no reference vectors exist for flow control).
 """
@@ -145,4 +149,103 @@ def explore(hops: int, nslots: int, steps: int, lines: int = 1, post_early: bool
             if nxt not in seen_states:
                 seen_states.add(nxt)
                 todo.append(nxt)
+    return res
+
+
+def explore_temporal(world: int, nslots: int, steps: int, handover: bool = True,
+                     max_states: int = 4_000_000) -> Result:
+    """The temporal allgather (``mintccl_amd/csrc/temporal.hpp``): ``world``
+    phases, phase c a broadcast of row c from rank c round the ring; one agent
+    per *position* that serves, in phase c, the rank c + position.  Steps are
+    numbered through the phases; a rank has ``nslots`` slots and one credit
+    word, which a different agent posts in every phase.  ``handover`` is the
+    rule that makes that safe: before its first post of a phase an agent waits
+    until the word has reached the phase's first step (the origin, whose
+    rank's slots stay empty, posts the whole phase at its end and waits
+    there).  Without it an agent can publish a later count while the agent
+    that served the rank before has not emptied its last slots - the checker
+    must report that as ``overwritten`` (or as the deadlock a count that went
+    backwards leads to)."""
+    S = steps
+
+    def need(gs: int) -> int:
+        return max(0, gs - nslots + 1)
+
+    programs = []
+    for h in range(world):
+        prog = []
+        for c in range(world):
+            rank, nxt, base = (c + h) % world, (c + h + 1) % world, c * S
+            if h and handover and base:
+                prog.append(("wait_tail", rank, base))
+            for s in range(S):
+                gs = base + s
+                if h == 0:
+                    prog += [("wait_tail", nxt, need(gs)), ("write", nxt, gs)]
+                else:
+                    prog += [("poll", rank, gs), ("post", rank, gs + 1)]
+                    if h < world - 1:
+                        prog += [("wait_tail", nxt, need(gs)), ("write", nxt, gs)]
+            if h == 0:
+                if handover and base:
+                    prog.append(("wait_tail", rank, base))
+                prog.append(("post", rank, base + S))
+        programs.append(prog)
+
+    # state: pc per agent; per rank the slots as (tag, taken); per rank the credit word
+    init = (tuple(0 for _ in range(world)),
+            tuple(tuple((0, True) for _ in range(nslots)) for _ in range(world)),
+            tuple(0 for _ in range(world)))
+    res = Result()
+    seen_states = {init}
+    todo = deque([init])
+    while todo:
+        st = todo.popleft()
+        res.states += 1
+        if res.states > max_states:
+            raise RuntimeError("state space larger than max_states")
+        pc, slots, tail = st
+        succ = []
+        for h in range(world):
+            if pc[h] >= len(programs[h]):
+                continue
+            kind, r, x = programs[h][pc[h]]
+            nslots_r, ntail, bad = slots, tail, None
+            if kind == "wait_tail":
+                if tail[r] < x:
+                    continue
+            elif kind == "poll":
+                tag, taken = slots[r][x % nslots]
+                if tag != x + 1:
+                    continue
+                if taken:
+                    bad = "wrong"           # taken twice
+                row = list(slots[r]); row[x % nslots] = (tag, True)
+                nslots_r = slots[:r] + (tuple(row),) + slots[r + 1:]
+            elif kind == "write":
+                tag, taken = slots[r][x % nslots]
+                if not taken:
+                    bad = "over"
+                row = list(slots[r]); row[x % nslots] = (x + 1, False)
+                nslots_r = slots[:r] + (tuple(row),) + slots[r + 1:]
+            else:                           # post: a plain store, it may also lower the word
+                ntail = tail[:r] + (x,) + tail[r + 1:]
+            npc = pc[:h] + (pc[h] + 1,) + pc[h + 1:]
+            succ.append(((npc, nslots_r, ntail), bad))
+        if not succ:
+            if all(pc[h] >= len(programs[h]) for h in range(world)):
+                res.finals += 1
+            else:
+                res.deadlocks += 1
+            continue
+        for nxt_state, bad in succ:
+            if bad == "over":
+                res.overwritten += 1
+                continue
+            if bad == "wrong":
+                res.wrong += 1
+                continue
+            if nxt_state not in seen_states:
+                seen_states.add(nxt_state)
+                todo.append(nxt_state)
     return res

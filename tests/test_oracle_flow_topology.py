@@ -29,6 +29,23 @@ def test_checker_reports_a_lost_line_as_a_deadlock():
     assert r.deadlocks > 0 and r.finals == 0
 
 
+@pytest.mark.parametrize("world,nslots,steps", [
+    (2, 2, 3), (3, 2, 2), (3, 3, 2), (3, 2, 4), (4, 2, 2), (4, 3, 2), (5, 2, 1), (5, 3, 2)])
+def test_temporal_allgather_hands_its_credit_words_over_safely(world, nslots, steps):
+    """One agent per position; the rank it serves changes from phase to phase
+    and with it who posts a rank's credit word."""
+    r = flowmodel.explore_temporal(world, nslots, steps)
+    assert r.overwritten == 0 and r.wrong == 0 and r.deadlocks == 0 and r.finals == 1
+
+
+def test_checker_catches_a_credit_word_posted_without_the_hand_over():
+    # an agent that posts a rank's word before the agent that served the rank
+    # in the phase before is through releases slots that are still full
+    for world, nslots, steps in ((3, 2, 2), (3, 2, 3), (4, 2, 1)):
+        r = flowmodel.explore_temporal(world, nslots, steps, handover=False)
+        assert r.overwritten > 0
+
+
 def random_topology(n, rng, p=0.8):
     topo = {i: [] for i in range(n)}
     for a, b in itertools.combinations(range(n), 2):
