@@ -110,18 +110,17 @@ class Timer:
 
 
 # Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
-# step.  Alltoall: 6 slots, 2560 wavefronts in all (Simple protocol: 2 slots,
-# 5760 wavefronts).  Everything else: 3 slots
-# of 512 KiB, 4608
-# wavefronts (reducescatter: 3 slots of 448 KiB, 56 wave-channels per
-# (row, hop) instead of 64: 1.5 - 2 % faster; broadcast and allgather with CUs
-# set apart for their origins, tuned_origin_cus);
-# a slot may grow to TUNED_SLOT_BUDGET bytes when there are few hops.  The
-# reducing collectives, sendrecv and alltoall run thread blocks of 2
-# wave-channels (TUNED_THREADS_REDUCING; sendrecv -9 %, alltoall -7 % against
-# blocks of 4; broadcast the same either way, allgather 7 % slower) unless
-# the caller names a block size.  Staging is allocated for TUNED_NSLOTS slots of
-# TUNED_SLOT_BUDGET either way.
+# step.  3 slots of 512 KiB and 4608 wavefronts, with these exceptions:
+# reducescatter 3 slots of 448 KiB, 56 wave-channels per (row, hop) instead of
+# 64 (1.5 - 2 % faster); an LL128 sendrecv over one hop 4 slots of 1.5 MiB;
+# alltoall 6 slots and 2560 wavefronts in all under LL128, 2 slots and 5760
+# under Simple.  A slot may grow to TUNED_SLOT_BUDGET bytes when there are few
+# hops.  Sendrecv, broadcast, allgather and alltoall set compute units apart
+# for their origins (tuned_origin_cus).  The reducing collectives, sendrecv and
+# alltoall run thread blocks of 2 wave-channels (TUNED_THREADS_REDUCING;
+# sendrecv -9 %, alltoall -7 % against blocks of 4; broadcast the same either
+# way, allgather 7 % slower) unless the caller names a block size.  Staging is
+# allocated for TUNED_NSLOTS slots of TUNED_SLOT_BUDGET either way.
 TUNED_TOTAL_WAVES = 4608
 TUNED_SLOT_BLOCKS = 512
 TUNED_SLOT_BLOCKS_REDUCESCATTER = 448
