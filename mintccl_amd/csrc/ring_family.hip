@@ -36,6 +36,24 @@ int resident_blocks_per_cu(Kernel kernel, int threads, size_t lds_bytes) {
     return per_cu < 1 ? 1 : per_cu;
 }
 
+// Launch a plan whose grid fits `capacity` blocks.  Compute units set apart for
+// origins need a larger grid (blocks with nothing to do fill the rounds): where
+// that one does not fit and the plain one does, the plain order runs.
+inline int launch_resident(void (*kernel)(const RingArgs), const Plan& plan, int capacity,
+                           hipStream_t stream) {
+    if (plan.blocks <= capacity) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
+                           plan.args);
+        return launch_status();
+    }
+    if (!plan.args.origin_cus || plan.blocks_plain > capacity) return MINT_ERR_RESIDENCY;
+    RingArgs plain = plan.args;
+    plain.origin_cus = 0;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks_plain), dim3((unsigned)plan.threads), 0,
+                       stream, plain);
+    return launch_status();
+}
+
 // Own rows through LDS (reducing element types only): WPB wave-channels and
 // one fetcher wavefront per thread block, R groups in flight per wave-channel.
 template <int DT, int CP>
@@ -94,18 +112,7 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
     }
     int ncu = cus.load(std::memory_order_relaxed);
     if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    if (plan.blocks > per_cu * ncu) {
-        // CUs set apart for origins need a larger grid: without, if that fits
-        if (!plan.args.origin_cus || plan.blocks_plain > per_cu * ncu) return MINT_ERR_RESIDENCY;
-        RingArgs plain = plan.args;
-        plain.origin_cus = 0;
-        hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks_plain), dim3((unsigned)plan.threads),
-                           0, stream, plain);
-        return launch_status();
-    }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
-                       plan.args);
-    return launch_status();
+    return launch_resident(kernel, plan, per_cu * ncu, stream);
 }
 
 template <int PROTO, int DT>
@@ -133,10 +140,7 @@ int launch_tree(const Plan& plan, hipStream_t stream) {
     }
     int ncu = cus.load(std::memory_order_relaxed);
     if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
-                       plan.args);
-    return launch_status();
+    return launch_resident(kernel, plan, per_cu * ncu, stream);
 }
 
 // Allgather, temporal schedule (LL128, bytes): one wavefront per (rank,
@@ -155,10 +159,7 @@ int launch_temporal(const Plan& plan, hipStream_t stream) {
     }
     int ncu = cus.load(std::memory_order_relaxed);
     if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)plan.threads), 0, stream,
-                       plan.args);
-    return launch_status();
+    return launch_resident(kernel, plan, per_cu * ncu, stream);
 }
 
 template <int DT>

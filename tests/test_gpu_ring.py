@@ -701,6 +701,22 @@ def test_origin_cus_that_would_not_be_resident_fall_back_to_the_plain_order(dev)
     comm.check()
     want = torch.stack([host[r][r] for r in range(world)])
     assert all(torch.equal(b.cpu(), want) for b in bufs)
+    # the same for the temporal schedule and the tree at the tuned geometry
+    tuned = make_comm(world, origin_cus=20)
+    bufs = [h.to(dev) for h in host]
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    d = tuned.make_op(_lib.OP_ALLGATHER_TEMPORAL, _lib.BYTES, n, ptrs, ptrs, list(range(world)) + [0],
+                      row_stride=n)
+    tuned.launch(d)
+    tuned.check()
+    assert all(torch.equal(b.cpu(), want) for b in bufs)
+    bufs = [h.to(dev) for h in host]
+    ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+    d = tuned.make_op(_lib.OP_TREE_BROADCAST, _lib.BYTES, world * n, {0: ptrs[0]},
+                      {r: p for r, p in ptrs.items() if r}, list(range(world)) + [0], root=0)
+    tuned.launch(d)
+    tuned.check()
+    assert all(torch.equal(b.cpu(), host[0]) for b in bufs)
 
 
 @pytest.mark.parametrize("op", ["broadcast", "allgather", "sendrecv"])
