@@ -45,7 +45,10 @@ typedef enum {
     MINT_ERR_TOO_LARGE = -6,  /* a row does not fit a 32-bit offset window; or, for
                                  mint_ring_launch_static, the geometry does not fit
                                  the library's static scratch array */
-    MINT_ERR_STAGING = -7     /* staging_bytes is smaller than mint_ring_staging_bytes() */
+    MINT_ERR_STAGING = -7,    /* staging_bytes is smaller than mint_ring_staging_bytes() */
+    MINT_ERR_NOT_READY = -8   /* mint_ring_launch_static on a stream under capture before the
+                                 library has looked up its static array on this device:
+                                 call mint_static_init() (or one launch) first */
 } mint_error;
 
 typedef enum { MINT_LAYOUT_PAIR = 0, MINT_LAYOUT_WAVE64 = 1 } mint_layout;
@@ -107,7 +110,13 @@ typedef enum {
  * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
  * that gave up; word 2: step it waited for; word 3: abort flag polled by all
  * other waits.  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
- * then holds that number.
+ * then holds that number.  Error code 3: MINT_PLACE_LOCAL, and the device did
+ * not deal the thread blocks evenly over its XCDs and compute units, so some
+ * (channel, position) found no block: nothing has been stored into any input
+ * or output buffer (a position waits for all seats to be taken before its
+ * first such store), and the same launch with MINT_PLACE_SPREAD (cache_policy
+ * 0) will do; after code 2 or 3 the staging is zeroed before it is used again
+ * (the launch left seat counters behind).
  * The words stay set until the caller zeroes them: every launch that finds
  * word 3 set gives up at its first wait (after at most 64 polls) and leaves
  * unspecified output, and only the first failure is recorded.  After a
@@ -193,8 +202,23 @@ typedef struct {
     uint32_t reserved1;    /* 0 */
 } mint_ring_op;
 
-/* 100 * major + minor of the descriptor layout: 101 = mint_ring_op with origin_cus. */
+/* 100 * major + minor of this interface: 102 = mint_build_flags, mint_static_init,
+ * mint_step_mix_deep, mint_ring_seat; mint_epoch_advance takes the protocol;
+ * every rank's staging grew by the seat tickets (101 = mint_ring_op with origin_cus).  A binding checks it against the
+ * version it was written for before it passes a descriptor. */
 int mint_version(void);
+/* What the library was compiled with, as bits.  A product build returns 0.
+ *   MINT_BUILD_RING_STATS   -DMINT_RING_STATS: the ring kernels collect wait
+ *                           accounting (mint_ring_debug.stats); results are right,
+ *                           times a few per cent longer
+ *   MINT_BUILD_ROW_NOLOAD   -DMINT_ROW_NOLOAD: whole blocks of the callers' rows
+ *                           are not loaded (their block numbers travel instead):
+ *                           WRONG RESULTS BY DESIGN, for timing a collective
+ *                           without its reads from HBM
+ * No counterpart in the reference. */
+#define MINT_BUILD_RING_STATS 1
+#define MINT_BUILD_ROW_NOLOAD 2
+int mint_build_flags(void);
 const char* mint_strerror(int err);
 
 /* Compute units, XCDs and wavefront size of the current device (the reference
@@ -252,6 +276,23 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
 int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
                   int waves, int iters, int what, void* sink, void* stream);
 
+/* mint_step_mix with several steps in flight per wavefront.  mint_step_mix has
+ * one: a step's loads are waited for and its store is issued before the next
+ * step's loads go out, so its time is steps x (load latency + store latency)
+ * and need not be what the device can do with the mix.  Here (`what` bits 1,
+ * 2, 4 as above) the loads run `ahead` = 1..3 steps ahead of their use and go
+ * out before the store of the step in hand: ahead + 1 steps of loads in flight
+ * per wavefront, the stores never waited for.  A wavefront owns ahead + 2 slots
+ * of 1 KiB in `staging` (needs waves * (ahead + 2) * 1024 bytes); with
+ * `partner` != 0 it loads what the same wavefront of the thread block 8
+ * further on stores (the same XCD, another compute unit - a line is written
+ * by one compute unit and read by another, as in a ring), else what it stored
+ * itself ahead + 1 steps earlier.  `iters` is a multiple of ahead + 1.  No
+ * counterpart in the reference. */
+int mint_step_mix_deep(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
+                       int waves, int iters, int what, int ahead, int partner, void* sink,
+                       void* stream);
+
 /* Standalone LL128 codec (load_ll128 + send_ll128 / recv_ll128 + save_ll128,
  * protocol.py:57-137).  Line L (0-based) carries flag_base + L * flag_stride:
  * MINT_LAYOUT_PAIR is the reference's wire format (120 payload bytes, then the
@@ -291,6 +332,22 @@ int mint_ring_grid_blocks(const mint_ring_op* op);
 int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int wave,
                        uint32_t max_entries, uint32_t* step, uint32_t* block,
                        uint32_t* recv_offset, uint32_t* send_offset, uint32_t* n_entries);
+/* Which seat a thread block takes under MINT_PLACE_LOCAL, computed on the host
+ * by the code the kernels run.  The reference maps program_id to its work
+ * directly (7_reducescatter.py:23-25: every rank is a GPU of its own); here a
+ * block claims an entry of the list of the XCD it finds itself on: the
+ * compute unit that was the `cu_rank`-th of XCD `xcd` to show up takes, with
+ * its `nth` block (0-based), entry nth * 32 + cu_rank; blocks beyond a compute
+ * unit's share and compute units beyond the 32nd draw a leftover ticket
+ * (`leftover` = the ticket such a block would be handed; *used_leftover says
+ * whether it was).  A launch of at most 32 entries per XCD (no compute unit
+ * gets a second block) takes the whole list by that ticket.  Returns 1 and the seat (pipeline, position, block of the
+ * position's group of thread blocks), 0 if the block has nothing to do, or a
+ * negative mint_error.  Needs no GPU: the test of "every seat exactly once
+ * for any arrival order". */
+int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, int leftover,
+                   int* used_leftover, int* pipeline, int* position, int* block_of_group);
+
 /* Validate and enqueue one fused launch that runs every rank's kernel: the
  * Triton launches kernel[(NUM_BLOCKS,)](recvbuff, sendbuff, inputbuff,
  * outputbuff, count, ...) of 2_sendrecv_indirect.py:165-166,
@@ -328,30 +385,45 @@ int mint_ring_launch_debug(const mint_ring_op* op, const mint_ring_debug* dbg, v
  * nslots * slot_bytes > MINT_STATIC_SLOT_BYTES or with more than
  * MINT_STATIC_CHANNELS wave-channels per rank (pipelines x phases x
  * waves_per_channel_group) is refused with MINT_ERR_TOO_LARGE.
- * The call enqueues, on `stream`, a kernel that advances the epoch kept in the
- * array (and clears the array when the 12-bit count starts over), a clearing
- * kernel when an LL128 launch follows a Simple one, and the ring launch; it
- * calls no hipMalloc / hipFree and no allocating library routine.  All calls
- * on a GPU share that GPU's array: two calls that overlap in time on one GPU
- * (different streams, or threads) race - keep them on one stream.  The first
- * call on a device looks the array's address up (hipGetSymbolAddress) with
- * that device current. */
+ * The call enqueues, on `stream`, a one-block kernel that advances the epoch
+ * kept in the array and the ring launch; it calls no hipMalloc / hipFree and no
+ * allocating library routine.  The epoch kernel clears the array (a fill of
+ * its own, no memset) on first use, when the 12-bit count starts over, and when
+ * an LL128 launch follows a Simple one - which it decides on the device, from
+ * a word in the array that holds the protocol of the launch before, so a
+ * launch captured into a graph decides anew at every replay, whatever ran
+ * between the replays.  All calls on a GPU share that GPU's array: two calls
+ * that overlap in time on one GPU (different streams, or threads) race - keep
+ * them on one stream.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress) with that device current; a stream under capture is
+ * no place for that, so a caller that captures calls mint_static_init() on
+ * the device beforehand (MINT_ERR_NOT_READY otherwise). */
 #define MINT_STATIC_SCRATCH_BYTES (16u << 20)
 #define MINT_STATIC_HEADER_BYTES 4096u
 #define MINT_STATIC_RANK_BYTES ((MINT_STATIC_SCRATCH_BYTES - MINT_STATIC_HEADER_BYTES) / MINT_MAX_RANKS)
 #define MINT_STATIC_CHANNELS 1024u
-#define MINT_STATIC_SLOT_BYTES (MINT_STATIC_RANK_BYTES - MINT_STATIC_CHANNELS * 256u)
+#define MINT_STATIC_SLOT_BYTES (MINT_STATIC_RANK_BYTES - MINT_STATIC_CHANNELS * 256u - 32768u)
 int mint_ring_launch_static(const mint_ring_op* op, void* stream);
+/* Looks up the address of the static array on the current device (once; later
+ * calls return at once).  Enqueues nothing and allocates nothing.  For callers
+ * of mint_ring_launch_static that capture their first launch. */
+int mint_static_init(void);
 
 /* Advances the epoch word a mint_ring_op points to with epoch_ptr (device
  * uint32, zero before its first use): 1, 2, ..., 4095, 1, ...  Whenever the
  * count starts over (and on first use) the kernel also zeroes
  * staging[0, staging_bytes) - the whole staging allocation of all ranks - as
- * the epoch contract demands.  Enqueued on `stream` like a launch; it is what
- * makes a captured sequence of collectives replayable, because a replay then
- * sees fresh epochs.  No counterpart in the reference (its flags restart with
- * every launch and it clears nothing). */
-int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, void* stream);
+ * the epoch contract demands.  `protocol` = -1, or the mint_protocol of the
+ * launch that follows: then `epoch_word` points to TWO uint32 (both zero
+ * before their first use), the second remembers the protocol of the launch
+ * before, and the staging is also cleared when an LL128 launch follows a
+ * Simple one on it (raw payload of a Simple launch could pass for LL128 sector
+ * tags).  Enqueued on `stream` like a launch; it is what makes a captured
+ * sequence of collectives replayable, because a replay then sees fresh epochs
+ * and takes the clearing decision itself, on the device.  No counterpart in the
+ * reference (its flags restart with every launch and it clears nothing). */
+int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, int protocol,
+                       void* stream);
 
 /* Torn-line probe: `pairs` producer wavefronts each rewrite 1 KiB blocks of
  * their own `iters` times; every 64-byte sector carries a tag and a payload

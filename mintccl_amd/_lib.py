@@ -25,7 +25,10 @@ STATUS_WORDS = 4
 MAX_EPOCH = 4095          # sector tags carry a 12-bit launch epoch
 
 (OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE,
- ERR_STAGING) = 0, -1, -2, -3, -4, -5, -6, -7
+ ERR_STAGING, ERR_NOT_READY) = 0, -1, -2, -3, -4, -5, -6, -7, -8
+VERSION = 102             # the interface version this binding was written for
+TICKET_BYTES = 18 * 1024  # the end of every rank's staging: room for the seat tickets
+BUILD_RING_STATS, BUILD_ROW_NOLOAD = 1, 2
 LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
 F16, BF16, F32, BYTES = 0, 1, 2, 3
 PROTO_LL128, PROTO_SIMPLE = 0, 1
@@ -85,12 +88,14 @@ _opp = ctypes.POINTER(RingOp)
 _dbgp = ctypes.POINTER(RingDebug)
 SYMBOLS = {
     "mint_version": (_i, []),
+    "mint_build_flags": (_i, []),
     "mint_strerror": (ctypes.c_char_p, [_i]),
     "mint_device_info": (_i, [_ip, _ip, _ip]),
     "mint_xcd_map": (_i, [_i, _vp, _vp]),
     "mint_copy_simple": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "mint_read_xor": (_i, [_vp, _sz, _vp, _i, _i, _vp]),
     "mint_step_mix": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _vp, _vp]),
+    "mint_step_mix_deep": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _i, _i, _vp, _vp]),
     "mint_ll128_packed_bytes": (_sz, [_sz, _i]),
     "mint_ll128_pack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp]),
     "mint_ll128_unpack": (_i, [_vp, _vp, _sz, _u64, _u64, _i, _vp, _vp]),
@@ -98,10 +103,12 @@ SYMBOLS = {
     "mint_ring_staging_bytes": (_sz, [_opp]),
     "mint_ring_grid_blocks": (_i, [_opp]),
     "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
+    "mint_ring_seat": (_i, [_opp, _i, _i, _i, _i, _ip, _ip, _ip, _ip]),
     "mint_ring_launch": (_i, [_opp, _vp]),
     "mint_ring_launch_debug": (_i, [_opp, _dbgp, _vp]),
     "mint_ring_launch_static": (_i, [_opp, _vp]),
-    "mint_epoch_advance": (_i, [_vp, _vp, _sz, _vp]),
+    "mint_static_init": (_i, []),
+    "mint_epoch_advance": (_i, [_vp, _vp, _sz, _i, _vp]),
     "mint_torn_line_probe": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _u32, _u32, _vp, _vp]),
 }
 
@@ -129,10 +136,10 @@ def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | N
     The ring kernels are one translation unit per element type; the five
     compilations run side by side and are linked at the end.  ``defines``
     (``-DMINT_RING_STATS``: wait accounting per ring position,
-    ``-DMINT_EARLY_POLL_ALL``: the adding kernels poll a step ahead like the
-    copying ones, ``-DMINT_ROW_NOLOAD``: whole blocks of own rows are not
-    loaded - wrong results, for timing a collective without its HBM reads) and ``so_path`` make a diagnostic build beside the product's;
-    ``MINTCCL_LIBRARY`` loads it."""
+    ``-DMINT_ROW_NOLOAD``: whole blocks of own rows are not loaded - wrong
+    results, for timing a collective without its HBM reads) and ``so_path``
+    make a diagnostic build beside the product's; ``MINTCCL_LIBRARY`` loads it,
+    ``mint_build_flags`` says which one is loaded."""
     out = so_path or os.path.join(_PKG, "libmintccl.so")
     build_dir = BUILD_DIR if so_path is None else out + ".objs"
     os.makedirs(build_dir, exist_ok=True)
@@ -188,11 +195,33 @@ def lib():
                 "(or mintccl_amd._lib.build()) in the repository root. "
                 "There is no CPU fallback.")
         L = ctypes.CDLL(SO_PATH)
+        # The descriptor below is laid out for one version of the interface: a
+        # stale or diagnostic library of another version would read it shifted.
+        L.mint_version.restype, L.mint_version.argtypes = ctypes.c_int, []
+        if L.mint_version() != VERSION:
+            raise RuntimeError(
+                f"{SO_PATH} speaks interface version {L.mint_version()}, this binding {VERSION}: "
+                "rebuild it (mintccl_amd._lib.build())")
         for name, (res, args) in SYMBOLS.items():
             fn = getattr(L, name)
             fn.restype, fn.argtypes = res, args
+        # A library that was built to return wrong results (timing without the
+        # reads of the rows) is only loaded by who asks for it by name.
+        flags = L.mint_build_flags()
+        if flags & BUILD_ROW_NOLOAD and os.getenv("MINTCCL_ALLOW_DIAGNOSTIC") != "1":
+            raise RuntimeError(
+                f"{SO_PATH} was built with -DMINT_ROW_NOLOAD and returns wrong results by design; "
+                "set MINTCCL_ALLOW_DIAGNOSTIC=1 to load it for timing")
         _lib = L
     return _lib
+
+
+def build_flags() -> list[str]:
+    """Names of the diagnostic switches the loaded library was built with
+    (empty for a product build)."""
+    flags = lib().mint_build_flags()
+    return [name for bit, name in ((BUILD_RING_STATS, "MINT_RING_STATS"),
+                                   (BUILD_ROW_NOLOAD, "MINT_ROW_NOLOAD")) if flags & bit]
 
 
 def check(code: int, where: str) -> None:

@@ -141,7 +141,9 @@ class RingTimeout(RuntimeError):
 
 class PlacementError(RuntimeError):
     """The local placement ran on a device that numbers its XCDs beyond 7
-    (status word 0 == 2)."""
+    (status word 0 == 2) or that did not deal the thread blocks evenly over
+    its XCDs and compute units (status word 0 == 3; no caller buffer has been
+    written then)."""
 
 
 def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
@@ -334,8 +336,13 @@ class VirtualComm:
         # and credit 0 mean "nothing yet" (2_sendrecv_indirect.py:59-60).
         if self.buff_size % 256:
             raise ValueError("staging size must be a multiple of 256 bytes")
-        self.rank_stride = self.buff_size + max(4096, self.slot_bytes // 4)
-        self.rank_stride = (self.rank_stride + 255) // 256 * 256
+        # (and the words thread blocks claim their seats through, behind them)
+        self.rank_stride = self.buff_size + max(4096, self.slot_bytes // 4) + _lib.TICKET_BYTES
+        # Whole multiples of 16 KiB between the ranks' staging: with ranks 18 or
+        # 20 KiB further apart than that the 8 x 256 MiB reduce-scatter takes 10 -
+        # 13 % longer (the slots of the ranks then fall differently onto the
+        # channels and sets of the L2 that holds them).
+        self.rank_stride = (self.rank_stride + 16383) // 16384 * 16384
         self.staging = torch.zeros(self.world_size * self.rank_stride, dtype=torch.uint8,
                                    device=self.device)
         self.status = torch.zeros(_lib.STATUS_WORDS, dtype=torch.int64, device=self.device)
@@ -348,7 +355,10 @@ class VirtualComm:
         # kernel that advances it (and clears staging when it starts over).
         if device_epoch is None:
             device_epoch = bool(os.getenv("MINTCCL_DEVICE_EPOCH", ""))
-        self.epoch_word = (torch.zeros(1, dtype=torch.int32, device=self.device)
+        # (two words: the epoch, and the protocol of the launch before - the
+        # kernel that advances the epoch also decides, on the device, whether
+        # an LL128 launch that follows a Simple one needs the slots cleared)
+        self.epoch_word = (torch.zeros(2, dtype=torch.int32, device=self.device)
                            if device_epoch else None)
         self._tls = threading.local()
         self._pending: dict = {}
@@ -498,8 +508,13 @@ class VirtualComm:
         # tags: payload left behind by a Simple launch could pass for the tags
         # of a later LL128 launch, so the slots are cleared (a stream-ordered
         # fill) when an LL128 launch follows a Simple one on this staging.
+        # With the epoch in device memory that decision is taken on the device
+        # (mint_epoch_advance is told the protocol), so that a launch captured
+        # into a graph takes it anew at every replay.  A launch on staging the
+        # caller brought (sendrecv_buffer) is the caller's to keep to one
+        # protocol or to clear.
         own_staging = d.staging[0] == self.staging_ptr(0)
-        if own_staging:
+        if own_staging and self.epoch_word is None:
             if d.protocol == _lib.PROTO_LL128 and self._last_protocol == _lib.PROTO_SIMPLE:
                 self.staging.zero_()
                 self.epoch = 0
@@ -525,7 +540,8 @@ class VirtualComm:
             if self.epoch_word is not None:
                 _lib.check(self._lib.mint_epoch_advance(
                     self.epoch_word.data_ptr(), self.staging.data_ptr(),
-                    self.staging.numel() * self.staging.element_size(), stream),
+                    self.staging.numel() * self.staging.element_size(),
+                    d.protocol if own_staging else -1, stream),
                     "mint_epoch_advance")
             if getattr(d, "debug", None) is not None:
                 _lib.check(self._lib.mint_ring_launch_debug(d, d.debug, stream),
@@ -543,10 +559,23 @@ class VirtualComm:
         if st[0] != 0:
             self.status.zero_()
             who = st[1]
+            if st[0] in (2, 3):
+                # a launch that could not seat all its blocks leaves its seat
+                # counters behind: start from cleared staging
+                self.staging.zero_()
+                self.epoch = 0
+                if self.epoch_word is not None:
+                    self.epoch_word.zero_()
             if st[0] == 2:
                 raise PlacementError(
                     f"a block ran on XCD {st[2]}: the local placement deals work to XCDs 0..7; "
                     "use placement spread (and cache_policy 0) on this device")
+            if st[0] == 3:
+                raise PlacementError(
+                    "the device did not deal the thread blocks evenly over its XCDs and compute "
+                    "units, so a (channel, position) of the local placement found no block; no "
+                    "input or output buffer has been written - run the launch again with "
+                    "placement spread (and cache_policy 0)")
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
                 f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]} "

@@ -35,22 +35,34 @@ __global__ void __launch_bounds__(1024) copy_simple_kernel(const uint8_t* __rest
 
 // Advances a launch epoch kept in device memory: 1, 2, ..., max_epoch, 1, ...
 // and clears the staging memory whenever it starts over, so that no sector
-// tag of an earlier launch with the same number survives.  One block: the
-// clearing happens once in max_epoch launches.
+// tag of an earlier launch with the same number survives.  With `track` the
+// word behind the epoch remembers the protocol of the launch before
+// (protocol + 1; 0 = none yet), and the memory is also cleared when an LL128
+// launch follows a Simple one: raw payload a Simple launch left in a slot could
+// pass for the sector tags an LL128 launch looks for.  The decision is taken
+// here, on the device, when the kernel runs - not on the host when the launch
+// is enqueued - so a launch that was captured into a graph decides anew at
+// every replay.  One block: the clearing is rare.
 __global__ void __launch_bounds__(1024) epoch_advance_kernel(uint32_t* epoch_word, uint8_t* staging,
                                                              uint64_t staging_bytes,
-                                                             uint32_t max_epoch) {
-    const uint32_t cur = *epoch_word;
+                                                             uint32_t max_epoch, uint32_t track,
+                                                             uint32_t protocol) {
+    const uint32_t cur = epoch_word[0];
+    const uint32_t before = track ? epoch_word[1] : 0u;
     __syncthreads();
     uint32_t next = cur + 1u;
-    if (cur == 0u || cur >= max_epoch) {      // first use, or the tags are about to repeat
+    const bool tags_forged = track && protocol == 0u /* LL128 */ && before == 2u /* Simple + 1 */;
+    if (cur == 0u || cur >= max_epoch || tags_forged) {   // first use, tags about to repeat, or forgeable
         const u32x4 zero = {0u, 0u, 0u, 0u};
         for (uint64_t i = threadIdx.x; i < (staging_bytes >> 4); i += blockDim.x)
             *reinterpret_cast<u32x4*>(staging + (i << 4)) = zero;
         next = 1u;
     }
     __syncthreads();
-    if (threadIdx.x == 0) *epoch_word = next;
+    if (threadIdx.x == 0) {
+        epoch_word[0] = next;
+        if (track) epoch_word[1] = protocol + 1u;
+    }
 }
 
 // Clears [p, p + nbytes), whole 16-byte vectors, with a grid-stride fill.  It
@@ -153,6 +165,92 @@ __global__ void __launch_bounds__(256) step_mix_kernel(const uint8_t* __restrict
         else if (!(WHAT & 16)) acc ^= x;
     }
     if (!(WHAT & 20) && acc.x == 0x9E3779B9u && acc.y == 0x85EBCA6Bu && acc.z == 0xC2B2AE35u)
+        sink[0] = acc.w;     // keeps the loads alive; practically never taken
+}
+
+// ---- the same traffic with several steps in flight per wavefront ---------------
+// step_mix_kernel above has one step in flight per wavefront: a step's loads
+// are issued, waited for, added and stored before the next step's loads go
+// out, and since a wavefront's vector-memory operations retire in issue order
+// every step also waits for the previous step's store.  Its time is therefore
+// (steps) x (a load's latency + a store's), which need not be what the device
+// can do with the mix.  Here the loads run AHEAD steps ahead of their use and
+// are older than the store of the step before them, so a wait for a step's
+// loads leaves the younger loads and every store in flight: AHEAD + 1 steps of
+// loads per wavefront, no store -> load chain inside a wavefront.
+// A wavefront owns AHEAD + 2 slots of 1 KiB; it stores step i into its slot
+// i mod (AHEAD + 2) and loads step j from slot (j + 1) mod (AHEAD + 2) of its
+// *partner* - the same wavefront of the thread block 8 further on (block ^ 8:
+// the same XCD, another CU), or itself (partner = 0) - which is what a ring
+// does to a line: written by one CU, read by another a step later.  Nothing is
+// synchronised; the values are whatever is there.
+//
+// The order of the memory operations is what is measured: a compiler fence and
+// a scheduling barrier stand between the phases of a step (the compiler, left
+// to itself, gathers the loads of an unrolled loop at its top and waits for
+// all of them); the waits are the compiler's own, which counts the operations
+// issued after the one it needs.
+__device__ __forceinline__ void mix_phase() {
+    compiler_fence();
+    __builtin_amdgcn_sched_barrier(0);
+    compiler_fence();
+}
+template <int WHAT, int AHEAD>
+__global__ void __launch_bounds__(256) step_mix_deep_kernel(const uint8_t* rows, uint8_t* staging,
+                                                            uint32_t staging_bytes,
+                                                            uint32_t waves, uint32_t iters,
+                                                            uint32_t partner, uint32_t* sink) {
+    constexpr uint32_t NS = AHEAD + 2;
+    const LaneMap m;
+    const uint32_t wpb = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * wpb + (uint32_t)wave_in_block());
+    if (wave >= waves) return;
+    uint32_t other = partner ? wave ^ (8u * wpb) : wave;
+    if (other >= waves) other = wave;
+    const Window win(staging, staging_bytes);
+    const uint32_t st_base = wave * NS * kBlockMsg + m.lane * 16u;
+    const uint32_t ld_base = other * NS * kBlockMsg + m.lane * 16u;
+    const uint32_t row_lane = m.flag_lane ? m.raw_off - 4u : m.raw_off;
+    u32x4 own[AHEAD + 1], got[AHEAD + 1];
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    uint32_t ld_slot = 1u, st_slot = 0u, ld_step = 0u;
+    // loads of one step; beyond the last step any valid address
+    auto issue = [&](int d) __attribute__((always_inline)) {
+        const uint32_t j = ld_step < iters ? ld_step : iters - 1u;
+        own[d] = got[d] = u32x4{0u, 0u, 0u, 0u};
+        if (WHAT & 1)
+            own[d] = __builtin_nontemporal_load((MINT_GLOBAL const u32x4_a1*)(
+                rows + (uint64_t)(j * waves + wave) * kBlockRawLL + row_lane));
+        if (WHAT & 2) got[d] = ld128<CP_SC1>(win, ld_base + ld_slot * kBlockMsg);
+        ld_slot = ld_slot + 1u == NS ? 0u : ld_slot + 1u;
+        ++ld_step;
+    };
+    // the prologue leaves the queue a later step finds (a store behind every
+    // step's loads): the compiler takes the smaller count where paths meet
+#pragma unroll
+    for (int d = 0; d <= AHEAD; ++d) {
+        if (WHAT & 4) st128<CP_NONE>(win, st_base + (uint32_t)d * kBlockMsg, acc);
+        mix_phase();
+        issue(d);
+        mix_phase();
+    }
+    for (uint32_t i = 0; i < iters; i += AHEAD + 1) {
+#pragma unroll
+        for (int d = 0; d <= AHEAD; ++d) {
+            // (the store first: the step's registers are free again when the
+            // loads that refill them are issued.  Either way the store is
+            // younger than the loads the next wait is for.)
+            const u32x4 x = add_rn<DT_F16>(own[d], got[d]);
+            mix_phase();
+            if (WHAT & 4) st128<CP_NONE>(win, st_base + st_slot * kBlockMsg, x);
+            else acc ^= x;
+            st_slot = st_slot + 1u == NS ? 0u : st_slot + 1u;
+            mix_phase();
+            issue(d);
+            mix_phase();
+        }
+    }
+    if (!(WHAT & 4) && acc.x == 0x9E3779B9u && acc.y == 0x85EBCA6Bu && acc.z == 0xC2B2AE35u)
         sink[0] = acc.w;     // keeps the loads alive; practically never taken
 }
 

@@ -17,13 +17,25 @@ using namespace mint;
 // loaded.  Every GPU the library runs on holds its own copy at its own
 // address.  In host code the name `scratch` only identifies the symbol; the
 // device address comes from hipGetSymbolAddress, once per device.
-//   [0, 4096)                              header: word 0 = launch epoch
+//   [0, 4096)                              header: word 0 = launch epoch, word 1 = protocol
+//                                          of the launch before (+ 1; 0 = none yet)
 //   4096 + r * MINT_STATIC_RANK_BYTES      rank r: [slots ... | credit words (last 256 KiB)]
 static __device__ __align__(256) unsigned char scratch[MINT_STATIC_SCRATCH_BYTES];
 
 namespace {
 
-constexpr int kVersion = 101;   // 0.1.1: mint_ring_op grew by origin_cus
+constexpr int kVersion = 102;   // 0.1.2: mint_build_flags, mint_static_init, mint_step_mix_deep,
+                                // mint_ring_seat; mint_epoch_advance takes the protocol; staging
+                                // grew by the seat tickets
+// What this library was compiled with (mint_build_flags).
+constexpr int kBuildFlags = 0
+#ifdef MINT_RING_STATS
+                            | MINT_BUILD_RING_STATS
+#endif
+#ifdef MINT_ROW_NOLOAD
+                            | MINT_BUILD_ROW_NOLOAD
+#endif
+    ;
 constexpr uint32_t kDefaultSpinBudget = 4000000u;
 constexpr uint32_t kMaxEpoch = 4095u;          // 12 bits of every sector tag
 constexpr uint32_t kMaxSteps = (1u << 20) - 1; // 20 bits of every sector tag
@@ -284,7 +296,22 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         }
     }
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
-    plan->staging_need = (size_t)a.credit_off + (size_t)a.shares * (size_t)a.waves * kCreditStride;
+    // Every rank's staging ends in room for the counters the blocks of a launch
+    // under the local placement claim their seats through (those of the first
+    // rank that has staging are used): at the end of what the caller
+    // allocated, so that launches of any geometry on the same staging find
+    // the same counters, never another launch's credit words.
+    const size_t credit_end = (size_t)a.credit_off + (size_t)a.shares * (size_t)a.waves * kCreditStride;
+    plan->staging_need = credit_end + kTicketBytes;
+    a.tickets = nullptr;
+    {
+        const size_t have = op->staging_bytes >= plan->staging_need ? (size_t)op->staging_bytes
+                                                                    : plan->staging_need;
+        const size_t ticket_off = (have - kTicketBytes) / 256 * 256;
+        for (int r = 0; r < op->world && !a.tickets; ++r)
+            if (op->staging[r]) a.tickets = reinterpret_cast<uint64_t*>(op->staging[r] + ticket_off);
+    }
+    if (op->placement == MINT_PLACE_LOCAL && !plan->empty && !a.tickets) return MINT_ERR_ARG;
     // The credit words lie behind the slots: a buffer that only holds the
     // slots (the reference's recvbuff is BUFF_SIZE bytes, 7_reducescatter.py:93)
     // would be written out of bounds.
@@ -312,22 +339,24 @@ constexpr size_t kStaticHeader = MINT_STATIC_HEADER_BYTES;
 constexpr size_t kStaticRank = MINT_STATIC_RANK_BYTES;
 constexpr size_t kStaticSlots = MINT_STATIC_SLOT_BYTES;
 static_assert(kStaticRank % 256 == 0 && kStaticSlots % 256 == 0, "credit words are 256-byte lines");
+static_assert(kStaticSlots + MINT_STATIC_CHANNELS * 256u + kTicketBytes <= kStaticRank, "seat tickets");
 static_assert(kStaticHeader + MINT_MAX_RANKS * kStaticRank <= MINT_STATIC_SCRATCH_BYTES, "layout");
 
 struct StaticScratch {
     std::atomic<unsigned char*> ptr{nullptr};   // device address of `scratch` on this device
-    std::atomic<int> last_protocol{-1};         // protocol of the previous launch on it
 };
 StaticScratch g_static[kMaxDevices];
 
 // Device address of this device's copy of `scratch` (looked up on the first
-// call with that device current).
-int static_scratch(int* dev_out, unsigned char** out) {
+// call with that device current; `may_look_up` = false refuses instead: a
+// stream under capture is no place for the look-up).
+int static_scratch(unsigned char** out, bool may_look_up = true) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return MINT_ERR_HIP;
     if (dev < 0 || dev >= kMaxDevices) return MINT_ERR_ARG;
     unsigned char* p = g_static[dev].ptr.load(std::memory_order_acquire);
     if (!p) {
+        if (!may_look_up) return MINT_ERR_NOT_READY;
         void* q = nullptr;
         if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) {
             (void)hipGetLastError();
@@ -336,7 +365,6 @@ int static_scratch(int* dev_out, unsigned char** out) {
         p = static_cast<unsigned char*>(q);
         g_static[dev].ptr.store(p, std::memory_order_release);
     }
-    *dev_out = dev;
     *out = p;
     return MINT_OK;
 }
@@ -377,6 +405,8 @@ extern "C" {
 
 int mint_version(void) { return kVersion; }
 
+int mint_build_flags(void) { return kBuildFlags; }
+
 const char* mint_strerror(int err) {
     switch (err) {
         case MINT_OK: return "ok";
@@ -387,6 +417,8 @@ const char* mint_strerror(int err) {
         case MINT_ERR_HIP: return "HIP runtime call failed";
         case MINT_ERR_TOO_LARGE: return "size does not fit the kernel's 32-bit counters";
         case MINT_ERR_STAGING: return "staging_bytes is smaller than mint_ring_staging_bytes()";
+        case MINT_ERR_NOT_READY:
+            return "first use on this device under stream capture: call mint_static_init() before";
         default: return "unknown error";
     }
 }
@@ -505,6 +537,36 @@ int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t sta
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), 0, as_stream(stream),
                        static_cast<const uint8_t*>(rows), static_cast<uint8_t*>(staging),
                        (uint32_t)staging_bytes, (uint32_t)waves, (uint32_t)iters,
+                       static_cast<uint32_t*>(sink));
+    return launch_status();
+}
+
+int mint_step_mix_deep(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
+                       int waves, int iters, int what, int ahead, int partner, void* sink,
+                       void* stream) {
+    if (waves <= 0 || iters <= 0 || what < 1 || what > 7 || ahead < 1 || ahead > 3)
+        return MINT_ERR_ARG;
+    if (iters % (ahead + 1)) return MINT_ERR_ARG;          // whole rounds of the unrolled loop
+    if ((what & 1) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
+        return MINT_ERR_ARG;
+    if ((size_t)waves * (size_t)iters >= (1ull << 32)) return MINT_ERR_TOO_LARGE;
+    const size_t need = (size_t)waves * (size_t)(ahead + 2) * kBlockMsg;
+    if ((what & 6) && (!staging || staging_bytes < need)) return MINT_ERR_ARG;
+    if ((what & 6) && staging_bytes >= (1ull << 31)) return MINT_ERR_TOO_LARGE;
+    if ((what & 6) && !aligned16(staging)) return MINT_ERR_ALIGN;
+    if (!(what & 4) && !sink) return MINT_ERR_ARG;
+    using Kernel = void (*)(const uint8_t*, uint8_t*, uint32_t, uint32_t, uint32_t, uint32_t,
+                            uint32_t*);
+#define MINT_DEEP_ROW(A)                                                                        \
+    {step_mix_deep_kernel<1, A>, step_mix_deep_kernel<2, A>, step_mix_deep_kernel<3, A>,        \
+     step_mix_deep_kernel<4, A>, step_mix_deep_kernel<5, A>, step_mix_deep_kernel<6, A>,        \
+     step_mix_deep_kernel<7, A>}
+    static const Kernel table[3][7] = {MINT_DEEP_ROW(1), MINT_DEEP_ROW(2), MINT_DEEP_ROW(3)};
+#undef MINT_DEEP_ROW
+    const unsigned blocks = ((unsigned)waves + 3u) / 4u;
+    hipLaunchKernelGGL(table[ahead - 1][what - 1], dim3(blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint8_t*>(rows), static_cast<uint8_t*>(staging),
+                       (uint32_t)staging_bytes, (uint32_t)waves, (uint32_t)iters, partner ? 1u : 0u,
                        static_cast<uint32_t*>(sink));
     return launch_status();
 }
@@ -637,6 +699,33 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
     }
 }
 
+int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, int leftover,
+                   int* used_leftover, int* pipeline, int* position, int* block_of_group) {
+    Plan plan;
+    const int err = make_plan(op, &plan);
+    if (err != MINT_OK) return err;
+    if (plan.empty || op->placement != MINT_PLACE_LOCAL || xcd < 0 || xcd >= kXcds || cu_rank < 0 ||
+        nth < 0 || leftover < 0)
+        return MINT_ERR_ARG;
+    const SeatList list = seat_list(plan.args, plan.blocks);
+    bool used = false;
+    int y;
+    if (seats_in_order_of_arrival(plan.args, list)) {
+        // taken in the order of arrival at one counter per XCD: `leftover` is that ticket
+        used = true;
+        y = leftover < list.len ? leftover : -1;
+    } else {
+        y = seat_entry(list, cu_rank, nth, leftover, used);
+    }
+    if (used_leftover) *used_leftover = used ? 1 : 0;
+    int p = 0, h = 0, gw = 0;
+    if (y < 0 || !seat_of_entry(plan.args, xcd, y, p, h, gw)) return 0;
+    if (pipeline) *pipeline = p;
+    if (position) *position = h;
+    if (block_of_group) *block_of_group = gw;
+    return 1;
+}
+
 int mint_ring_launch(const mint_ring_op* op, void* stream) {
     return mint_ring_launch_debug(op, nullptr, stream);
 }
@@ -665,41 +754,55 @@ int mint_ring_launch_static(const mint_ring_op* op, void* stream) {
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
 
-    int dev = 0;
+    // The array's address is looked up once per device.  Not while `stream` is
+    // being captured into a graph: the first call on a device then has to have
+    // happened before (mint_static_init).
+    hipStream_t s = as_stream(stream);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusNone;
+    }
     unsigned char* base = nullptr;     // device address; never the array's name
-    err = static_scratch(&dev, &base);
+    err = static_scratch(&base, capturing == hipStreamCaptureStatusNone);
     if (err != MINT_OK) return err;
     for (int r = 0; r < MINT_MAX_RANKS; ++r)
         plan.args.staging[r] = reinterpret_cast<uint64_t>(base + kStaticHeader + r * kStaticRank);
+    // (the seat tickets sit at the end of rank 0's part, as in make_plan)
+    plan.args.tickets = reinterpret_cast<uint64_t*>(
+        base + kStaticHeader + (reinterpret_cast<size_t>(plan.args.tickets) - 16));
     uint32_t* epoch_word = reinterpret_cast<uint32_t*>(base);
     plan.args.epoch_word = epoch_word;
 
     // The array keeps what the last call left in it.  The epoch in its first
     // word makes old sector tags and credit words meaningless to this launch;
-    // the kernel that advances it clears the array on first use and whenever
-    // the 12-bit count starts over.  Raw payload of a Simple launch could pass
-    // for LL128 tags, so the slots are cleared between the two (a fill
-    // kernel, which a caller may capture, not a memset).
-    hipStream_t s = as_stream(stream);
-    const int before = g_static[dev].last_protocol.exchange(op->protocol, std::memory_order_acq_rel);
-    if (op->protocol == MINT_PROTO_LL128 && before == MINT_PROTO_SIMPLE) {
-        hipLaunchKernelGGL(zero_kernel, dim3(256), dim3(256), 0, s, base + kStaticHeader,
-                           (uint64_t)(MINT_STATIC_SCRATCH_BYTES - kStaticHeader));
-        if ((err = launch_status()) != MINT_OK) return err;
-    }
+    // the kernel that advances it clears the array on first use, whenever the
+    // 12-bit count starts over, and when an LL128 launch follows a Simple one
+    // (raw payload of a Simple launch could pass for LL128 tags).  It takes
+    // that decision on the device from the protocol word beside the epoch, so
+    // a captured launch decides anew at every replay; the clearing is a fill
+    // by the kernel itself, not a memset node.
     hipLaunchKernelGGL(epoch_advance_kernel, dim3(1), dim3(1024), 0, s, epoch_word,
                        base + kStaticHeader, (uint64_t)(MINT_STATIC_SCRATCH_BYTES - kStaticHeader),
-                       kMaxEpoch);
+                       kMaxEpoch, 1u, (uint32_t)op->protocol);
     if ((err = launch_status()) != MINT_OK) return err;
     return launch_ring(plan, op->protocol, op->dtype, op->cache_policy, s);
 }
 
-int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, void* stream) {
+int mint_static_init(void) {
+    unsigned char* base = nullptr;
+    return static_scratch(&base);
+}
+
+int mint_epoch_advance(void* epoch_word, void* staging, size_t staging_bytes, int protocol,
+                       void* stream) {
     if (!epoch_word || (reinterpret_cast<uint64_t>(epoch_word) & 3u)) return MINT_ERR_ARG;
+    if (protocol < -1 || protocol > MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (staging_bytes && (!staging || !aligned16(staging) || staging_bytes % 16)) return MINT_ERR_ALIGN;
     hipLaunchKernelGGL(epoch_advance_kernel, dim3(1), dim3(1024), 0, as_stream(stream),
                        static_cast<uint32_t*>(epoch_word), static_cast<uint8_t*>(staging),
-                       (uint64_t)staging_bytes, kMaxEpoch);
+                       (uint64_t)staging_bytes, kMaxEpoch, protocol >= 0 ? 1u : 0u,
+                       protocol >= 0 ? (uint32_t)protocol : 0u);
     return launch_status();
 }
 

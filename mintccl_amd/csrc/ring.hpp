@@ -78,6 +78,7 @@ struct RingArgs {
     uint32_t origin_cus;                  // local placement: of the 32 CUs of an XCD, so many hold origins only (0: the plain order)
     uint64_t* stats;                      // optional: per position 8 x u64 of wait accounting
     uint32_t fetch_depth;                 // own rows through LDS: groups of LDS per wave-channel
+    uint64_t* tickets;                    // local placement: the words seats are claimed through (kTicket*)
 };
 
 struct Role {
@@ -159,6 +160,311 @@ __device__ __forceinline__ bool wait_count(const uint64_t* word, uint32_t epoch,
         if ((spins & 63u) == 63u && aborted(status)) return false;
         __builtin_amdgcn_s_sleep(2);
     }
+}
+
+// Which (pipeline, position, wave-channel) a wavefront serves.  `wpb` =
+// wave-channels per thread block, `wib` = this wavefront's index among them.
+constexpr int kCusPerXcd = 32;      // MI355X: 256 CUs in 8 XCDs
+struct Seat {
+    int p, h, gw, w;
+    uint32_t sequence;      // local placement: sequence number of the launch (seats_confirmed)
+    bool ok;
+};
+__device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int wib) {
+    // Index of a wave-channel inside its group: it decides which blocks of
+    // a step, which staging bytes and which credit word the wave owns.  Under
+    // the local placement the blocks of one XCD are numbered consecutively, so
+    // that what an XCD touches (staging, rows) is contiguous in memory instead
+    // of 4 KiB out of every 32: that spreads it over all channels and sets of
+    // that XCD's L2.
+    if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
+        return (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
+    return gw * wpb + wib;
+}
+
+// ---- seats under the local placement --------------------------------------------
+// XCD d serves the channels c with c % 8 == d: a channel's whole ring then
+// shares one L2.  The work of an XCD is a list of entries; entry y is one
+// (channel, position).  Which entry a thread block takes does not depend on
+// its number: the block asks the hardware where it runs (XCC_ID, and the
+// compute unit's number from HW_ID) and claims an entry through counters in
+// device memory.  Any order in which the device deals its blocks over XCDs
+// and compute units gives every entry to exactly one block, provided every
+// XCD receives an eighth of the grid and every compute unit its share of
+// that; if not, entries stay unclaimed, no position stores into a caller's
+// buffer (seats_confirmed below) and the launch reports status 3.
+//
+// The list of an XCD is walked in rounds of one entry per compute unit: the
+// compute unit that was the j-th of its XCD to show up takes, with its n-th
+// block, entry n * 32 + j.  All blocks of a compute unit so share j, and the
+// order of the list decides what a compute unit holds: with h = y % npos and
+// a position count that divides 32 (8 ranks) every compute unit holds blocks
+// of one position only - the positions that load from HBM sit on compute
+// units of their own and the polls of the others, answered by the L2, never
+// queue behind a load from HBM in a compute unit's memory pipeline.  The ring
+// walks are fastest that way (an allgather whose compute units hold a mix of
+// positions takes 4 - 10 % longer; the order in which blocks reach a counter
+// is nothing like the order of their numbers, so one counter per XCD would
+// mix them).  Entries of a last, partial round (a list that is no multiple of
+// 32) and blocks beyond a compute unit's share go through one more counter
+// per XCD, the leftover tickets.
+//
+// The counters (64-bit words in device memory, zero between launches):
+//   xcd * 2048 + cu * 8     per compute unit: blocks that have arrived in bits
+//                           23:0, j + 1 in bits 31:24 once it is known
+//   16384 + xcd * 128       per XCD, a line of its own: + 0 compute units
+//                           registered, + 8 leftover tickets handed out, + 16
+//                           entries claimed
+//   17408, 17416            XCDs whose list is claimed completely, for launches
+//                           of even / odd sequence number
+//   17536                   sequence number of the launch (a line of its own)
+// A line that blocks of several XCDs work on is slow (a counter per XCD in one
+// line: 40 - 60 us for 160 blocks per XCD; in lines of their own: 6 us), hence
+// the spacing.  The block that claims the last entry of its XCD's list puts
+// that XCD's counters back to zero, so a launch finds them as the launch
+// before left them - zero - and the common path is one atomic add per counter
+// (with the launch epoch in every word instead, every block of a launch found
+// a stale word first and went through a compare-and-swap: three more trips).
+// The count of complete XCDs is looked at long after it was counted up
+// (positions check it before their first store into a caller's buffer), so it
+// is not put back by its own launch: there are two, used in turn - the block
+// that counts the eighth XCD clears the other one and moves the sequence
+// number on, which every block reads when it starts.  A launch that could not
+// seat all its blocks (status 2 or 3) leaves counters behind: the staging is
+// cleared before it is used again.  All of these are atomics and loads at
+// agent scope: one place serves them whichever XCD asks.
+constexpr uint32_t kTicketXcdLine = 16384, kTicketXcdStride = 128, kTicketComplete = 17408,
+                   kTicketSequence = 17536;
+constexpr uint32_t kTicketBytes = 18 * 1024;
+constexpr uint32_t kSeatPatience = 1u << 18;
+
+// The list of one XCD: `len` entries, of which the first `full` rounds are
+// taken by (compute unit, arrival) and the `rest` after them by leftover ticket.
+struct SeatList {
+    int len, full, rest;
+};
+__host__ __device__ __forceinline__ SeatList seat_list(const RingArgs& a, int grid_blocks) {
+    SeatList l;
+    l.len = grid_blocks / kXcds;
+    l.full = l.len / kCusPerXcd;
+    l.rest = l.len % kCusPerXcd;
+    return l;
+}
+// Entry for the block that arrived `nth` on the compute unit registered as
+// `j`-th of its XCD; `leftover` = the ticket it would get from the XCD's
+// leftover counter, `used` says whether it took it.  -1: nothing to claim.
+__host__ __device__ __forceinline__ int seat_entry(const SeatList& l, int j, int nth, int leftover,
+                                                   bool& used) {
+    used = false;
+    if (j < kCusPerXcd && nth < l.full) return nth * kCusPerXcd + j;
+    used = true;
+    return leftover < l.rest ? l.full * kCusPerXcd + leftover : -1;
+}
+// A list of at most one round (a small launch: no compute unit gets a second
+// block) is simply taken in the order in which the blocks reach one counter:
+// one atomic instead of three trips.  (Not so the longer lists of launches
+// whose position count does not divide the compute units anyway, like the 9 of
+// a reduce-scatter: taken in the order of arrival, the 8 x 256 MiB
+// reduce-scatter needs 8 % longer.)
+__host__ __device__ __forceinline__ bool seats_in_order_of_arrival(const RingArgs& a,
+                                                                   const SeatList& l) {
+    return l.full == 0;
+}
+// What entry y of XCD `xcd` is: pipeline, position, block of the group.
+__host__ __device__ __forceinline__ bool seat_of_entry(const RingArgs& a, int xcd, int y, int& p,
+                                                       int& h, int& gw) {
+    const int npos = a.hops + 1;
+    // seat_turn turns the positions by two after every round over the compute
+    // units, which mixes them: the tree gains 10 % from that
+    int q = y / npos;
+    h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
+    if (a.origin_cus) {
+        // Origins on compute units of their own, and on more of them than
+        // their share of the blocks: in every round origin_cus of the compute
+        // units take an origin, the others take the receiving positions of the
+        // channels in turn.  Entries left over in either list are empty.
+        // (What a compute unit's memory pipeline keeps in flight is bounded;
+        // loads from HBM under a collective's stores take 2.5 us, so a
+        // compute unit full of origins delivers 10 GB/s and an eighth of them
+        // cannot feed the rest: allgather 8 x 128 MiB 3.4 ms, 1.9 ms without
+        // its loads.)
+        const int round = y / kCusPerXcd, j = y % kCusPerXcd, o = (int)a.origin_cus;
+        const int groups = a.pipes * a.blocks_per_group / kXcds;
+        // the origins' compute units lie evenly among the 32: `before` of them below j
+        const int before = j * o / kCusPerXcd;
+        if ((j + 1) * o / kCusPerXcd > before) {
+            q = round * o + before;
+            h = 0;
+        } else {
+            const int r = round * (kCusPerXcd - o) + (j - before);
+            q = r / (npos - 1);
+            h = 1 + r % (npos - 1);
+        }
+        if (q >= groups) return false;
+    }
+    const int c = q * kXcds + xcd;
+    p = c / a.blocks_per_group;
+    gw = c % a.blocks_per_group;
+    return true;
+}
+
+__device__ __forceinline__ uint32_t launch_epoch(const RingArgs& a) {
+    // The epoch normally is a launch argument; a caller that replays captured
+    // launches keeps it in device memory and advances it between launches.
+    return a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
+                              as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                        : a.epoch;
+}
+__device__ __forceinline__ uint64_t* ticket_word(const RingArgs& a, uint32_t byte_offset) {
+    return reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(a.tickets) + byte_offset);
+}
+__device__ __forceinline__ uint64_t ticket_add(uint64_t* word, uint64_t v) {
+    return __hip_atomic_fetch_add((MINT_GLOBAL unsigned long long*)word, (unsigned long long)v,
+                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// The entry of its XCD's list this thread block takes (called by one lane of
+// the block), or -1.  `xcd` comes back as the XCD it runs on, `last` says that
+// the block claimed the last entry of that XCD's list (it then puts the XCD's
+// counters back to zero: reset_tickets).  The wait here is for another block to
+// be dispatched, not for data: it gets at least kSeatPatience looks whatever
+// budget the caller gave the data waits.
+__device__ __forceinline__ int claim_entry(const RingArgs& a, uint32_t& sequence, int& xcd,
+                                           bool& last) {
+    last = false;
+    // (in flight together with the first atomic below)
+    const uint64_t seq_word = ld64_agent(ticket_word(a, kTicketSequence));
+    xcd = xcc_id();
+    if (xcd >= kXcds) {
+        report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
+        return -1;
+    }
+    const SeatList list = seat_list(a, (int)gridDim.x);
+    uint64_t* const line = ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride);
+    int y;
+    uint32_t claimed;
+    if (seats_in_order_of_arrival(a, list)) {
+        claimed = (uint32_t)ticket_add(line + 2, 1ull);
+        y = (int)claimed < list.len ? (int)claimed : -1;
+    } else {
+        // compute unit number inside the XCD: HW_ID bits 15:8 (CU, SH, SE)
+        const uint32_t cu = __builtin_amdgcn_s_getreg(4 | (8 << 6) | (7 << 11));
+        uint64_t* const word = ticket_word(a, (uint32_t)xcd * 2048u + cu * 8u);
+        const uint32_t before = (uint32_t)ticket_add(word, 1ull);
+        const uint32_t nth = before & 0xFFFFFFu;
+        uint32_t jfield = before >> 24;
+        if (before == 0u) {
+            // first block of this compute unit: register the unit, publish its j
+            jfield = (uint32_t)ticket_add(line, 1ull) + 1u;
+            if (jfield > 0xFFu) jfield = 0xFFu;
+            __hip_atomic_fetch_or((MINT_GLOBAL unsigned long long*)word,
+                                  (unsigned long long)jfield << 24, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            const uint32_t budget = a.spin_budget < kSeatPatience ? kSeatPatience : a.spin_budget;
+            for (uint32_t spins = 0; jfield == 0u; ++spins) {
+                if (spins >= budget) {
+                    report_error(a.status, 3, 0, 0, 0, (uint64_t)cu);
+                    return -1;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                jfield = ((uint32_t)ld64_agent(word) >> 24) & 0xFFu;
+            }
+            jfield &= 0xFFu;
+        }
+        bool wants_leftover;
+        y = seat_entry(list, (int)jfield - 1, (int)nth, 0, wants_leftover);
+        if (wants_leftover)
+            y = seat_entry(list, (int)jfield - 1, (int)nth, (int)ticket_add(line + 1, 1ull),
+                           wants_leftover);
+        if (y < 0) return -1;
+        claimed = (uint32_t)ticket_add(line + 2, 1ull);
+    }
+    sequence = (uint32_t)seq_word;
+    if (y < 0) return -1;
+    // the block that claims the last entry of its XCD says so to everybody; the
+    // one that does so for the last XCD prepares the counter of the next launch
+    if (claimed + 1u == (uint32_t)list.len) {
+        last = true;
+        uint64_t* const complete = ticket_word(a, kTicketComplete);
+        if (ticket_add(complete + (sequence & 1u), 1ull) + 1u == (uint64_t)kXcds) {
+            __hip_atomic_store((MINT_GLOBAL unsigned long long*)(complete + ((sequence & 1u) ^ 1u)), 0ull,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            (void)ticket_add(ticket_word(a, kTicketSequence), 1ull);
+        }
+    }
+    return y;
+}
+// Puts the counters of XCD `xcd` back to zero (the thread block that claimed
+// the last entry of the XCD's list; every other claim of the launch on this
+// XCD has been counted by then).
+__device__ __forceinline__ void reset_tickets(const RingArgs& a, int xcd) {
+    for (uint32_t i = threadIdx.x; i < 256u + 3u; i += blockDim.x) {
+        uint64_t* const w = i < 256u ? ticket_word(a, (uint32_t)xcd * 2048u + i * 8u)
+                                     : ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride) +
+                                           (i - 256u);
+        __hip_atomic_store((MINT_GLOBAL unsigned long long*)w, 0ull, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// Before a position stores into a caller's buffer for the first time: every
+// entry of every XCD's list has been claimed, so every (channel, position) of
+// the launch is being served.  Bounded; false (status 3) otherwise - then no
+// caller buffer has been written and the caller can run the launch again
+// with the spread placement.
+__device__ __forceinline__ bool seats_confirmed(const RingArgs& a, uint32_t sequence) {
+    if (a.placement != PLACE_LOCAL) return true;
+    const uint64_t* const word = ticket_word(a, kTicketComplete) + (sequence & 1u);
+    const uint32_t budget = a.spin_budget < kSeatPatience ? kSeatPatience : a.spin_budget;
+    for (uint32_t spins = 0;; ++spins) {
+        const uint32_t n = __builtin_amdgcn_readfirstlane((uint32_t)ld64_agent(word));
+        if (n == (uint32_t)kXcds) return true;
+        if (spins >= budget || ((spins & 63u) == 63u && aborted(a.status))) {
+            report_error(a.status, 3, 0, 0, 0, (uint64_t)n);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
+// The seat of this wavefront.  Under the local placement wavefront 0 of the
+// thread block claims the block's entry and hands it to the others through
+// `shared_entry` (two ints of LDS): every wavefront of the block has to call.
+__device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib, int wave_of_block,
+                                          MINT_LDS int* shared_entry) {
+    // (locals, not members of the result: a member passed by reference keeps
+    // the whole struct in scratch memory)
+    int p = 0, h = 0, gw = 0;
+    uint32_t sequence = 0;
+    bool seated = true;
+    if (a.placement == PLACE_LOCAL) {
+        if (wave_of_block == 0 && lane_id() == 0) {       // one lane: the counters count blocks
+            int xcd = 0;
+            bool last = false;
+            uint32_t seq = 0;
+            const int y = claim_entry(a, seq, xcd, last);
+            shared_entry[0] = y < 0 ? -1 : (y * kXcds + xcd) * 2 + (last ? 1 : 0);
+            shared_entry[1] = (int)(seq & 1u);
+        }
+        __syncthreads();
+        const int e = __builtin_amdgcn_readfirstlane(shared_entry[0]);
+        sequence = (uint32_t)__builtin_amdgcn_readfirstlane(shared_entry[1]);
+        if (e >= 0 && (e & 1)) reset_tickets(a, (e >> 1) % kXcds);
+        seated = e >= 0 && seat_of_entry(a, (e >> 1) % kXcds, (e >> 1) / kXcds, p, h, gw);
+    } else {
+        const int npos = a.hops + 1, x = (int)blockIdx.x;
+        const int c = x / npos;
+        h = x % npos;
+        p = c / a.blocks_per_group;
+        gw = c % a.blocks_per_group;
+    }
+    Seat st;
+    st.p = p; st.h = h; st.gw = gw; st.w = 0;
+    st.sequence = sequence;
+    st.ok = false;
+    if (!seated || gw * wpb + wib >= a.waves) return st;
+    st.w = seat_wave(a, gw, wpb, wib);
+    st.ok = !(h == 0 && a.skip_origin);
+    return st;
 }
 
 // ---- chunk scheduler --------------------------------------------------------
@@ -344,12 +650,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     uint64_t* nxt_tail = reinterpret_cast<uint64_t*>(a.staging[role.next] + nxt_chan);
     uint64_t* nxt_head = nxt_tail + 16;
 
-    // The epoch normally is a launch argument; a caller that replays captured
-    // launches keeps it in device memory and advances it between launches.
-    const uint32_t epoch =
-        a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
-                           as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-                     : a.epoch;
+    const uint32_t epoch = launch_epoch(a);
     const uint64_t flag_hi = (uint64_t)epoch << 32;        // credit / head words
     const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
     const uint32_t groups_per_step = K / U;
@@ -762,11 +1063,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         }
       }
     }
-#ifdef MINT_EARLY_POLL_ALL
-    if constexpr (PROTO == PROTO_LL128) {
-#else
     if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
-#endif
       if (!origin_done && K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
         uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
@@ -940,102 +1237,11 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     }
 }
 
-// Which (pipeline, position, wave-channel) a wavefront serves.  `wpb` =
-// wave-channels per thread block, `wib` = this wavefront's index among them.
-constexpr int kCusPerXcd = 32;      // MI355X: 256 CUs in 8 XCDs (a matter of speed only)
-struct Seat {
-    int p, h, gw, w;
-    bool ok;
-};
-__device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int wib) {
-    // Index of a wave-channel inside its group: it decides which blocks of
-    // a step, which staging bytes and which credit word the wave owns.  Under
-    // the local placement the blocks of one XCD are numbered consecutively, so
-    // that what an XCD touches (staging, rows) is contiguous in memory instead
-    // of 4 KiB out of every 32: that spreads it over all channels and sets of
-    // that XCD's L2.
-    if (a.placement == PLACE_LOCAL && a.blocks_per_group % kXcds == 0 && a.waves % wpb == 0)
-        return (gw % kXcds) * (a.waves / kXcds) + (gw / kXcds) * wpb + wib;
-    return gw * wpb + wib;
-}
-__device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib) {
-    Seat st;
-    st.ok = false;
-    st.p = st.h = st.gw = st.w = 0;
-    const int npos = a.hops + 1;
-    const int x = (int)blockIdx.x;
-    int c;
-    if (a.placement == PLACE_LOCAL) {
-        // Blocks are dealt round-robin over the XCDs, so every aligned group of
-        // 8 consecutive blocks lands on 8 different XCDs - but not always block
-        // x on XCD x % 8: which XCD block 0 goes to depends on the hardware
-        // queue the stream is mapped to (measured: 0 on a fresh process, 7 on
-        // the default stream once a second stream has been used).  So a block
-        // asks the hardware where it runs, and the group it belongs to says
-        // how far along that XCD's list of work it is: XCD d takes the
-        // channels c with c % 8 == d and its blocks walk through the
-        // positions of one channel after the other.  A channel's whole ring
-        // then shares one L2 by construction and is dispatched together.
-        const int xcd = xcc_id(), y = x / kXcds;
-        if (xcd >= kXcds) {
-            report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
-            return st;
-        }
-        //
-        // An XCD hands its blocks to its CUs in turn, so with h = y % npos and a
-        // position count that divides the CUs of an XCD (8 ranks) every CU
-        // holds blocks of one position only: the positions that load from HBM
-        // sit on CUs of their own and the polls of the others, answered by
-        // the L2, never queue behind a load from HBM in a CU's memory
-        // pipeline.  The ring walks are fastest that way (an allgather whose
-        // CUs hold a mix of positions takes 4 - 10 % longer).  The tree gains
-        // 10 % from a mix: seat_turn turns the positions by two after every
-        // round over the CUs.
-        int q = y / npos;
-        st.h = a.seat_turn ? (y % npos + (q / (int)a.seat_turn) * 2) % npos : y % npos;
-        if (a.origin_cus) {
-            // Origins on CUs of their own, and on more of them than their share
-            // of the blocks: the XCD's blocks are taken in rounds of one block
-            // per CU; in every round origin_cus of the CUs take an origin, the
-            // others take the receiving positions of the channels in turn.
-            // Blocks left over in either list have nothing to do.  (What a
-            // CU's memory pipeline keeps in flight is bounded, about 26 KB;
-            // loads from HBM under a collective's stores take 2.5 us, so a CU
-            // full of origins delivers 10 GB/s and an eighth of the CUs cannot
-            // feed the rest: allgather 8 x 128 MiB 3.4 ms, 1.9 ms without its
-            // loads.)
-            const int round = y / kCusPerXcd, j = y % kCusPerXcd, o = (int)a.origin_cus;
-            const int groups = a.pipes * a.blocks_per_group / kXcds;
-            // the origins' CUs lie evenly among the 32: `before` of them below CU j
-            const int before = j * o / kCusPerXcd;
-            if ((j + 1) * o / kCusPerXcd > before) {
-                q = round * o + before;
-                st.h = 0;
-            } else {
-                const int r = round * (kCusPerXcd - o) + (j - before);
-                q = r / (npos - 1);
-                st.h = 1 + r % (npos - 1);
-            }
-            if (q >= groups) return st;
-        }
-        c = q * kXcds + xcd;
-    } else {
-        st.h = x % npos;
-        c = x / npos;
-    }
-    st.p = c / a.blocks_per_group;
-    st.gw = c % a.blocks_per_group;
-    if (st.gw * wpb + wib >= a.waves) return st;
-    st.w = seat_wave(a, st.gw, wpb, wib);
-    st.ok = !(st.h == 0 && a.skip_origin);
-    return st;
-}
-
 // One specialised walk per role.
 template <int PROTO, int DT, int CPI, int U, bool LDSF>
-__device__ __forceinline__ void walk_as(const RingArgs& a, const Seat& st, const Role& role,
-                                        const LdsPort port = LdsPort{}) {
-    const int p = st.p, h = st.h, w = st.w, rk = role.rank, nx = role.next;
+__device__ __forceinline__ void walk_as(const RingArgs& a, const int p, const int h, const int w,
+                                        const Role role, const LdsPort port = LdsPort{}) {
+    const int rk = role.rank, nx = role.next;
     if (!role.recv) {
         ring_walk<PROTO, DT, CPI, U, LDSF>(a, p, h, w, FixedRole<true, false, false, false, true>{rk, nx}, port);
     } else if (role.reduce) {
@@ -1059,11 +1265,19 @@ template <int PROTO, int DT, int CPI, int U>
 __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     // the wave index is the same in every lane: keep it (and all the index
     // arithmetic that hangs off it) in scalar registers
+    __shared__ int entry[2];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
-    const Seat st = take_seat(a, wpb, wib);
+    const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
-    walk_as<PROTO, DT, CPI, U, false>(a, st, role_of(a, st.p, st.h));
+    // (plain integers from here on: a seat handed on by reference stays in
+    // scratch memory)
+    const int p = st.p, h = st.h, w = st.w;
+    const Role role = role_of(a, p, h);
+    // a position that writes a caller's buffer first makes sure that every
+    // (channel, position) of the launch has a thread block
+    if (role.save && !seats_confirmed(a, st.sequence)) return;
+    walk_as<PROTO, DT, CPI, U, false>(a, p, h, w, role);
 }
 
 // The fetcher wavefront of a thread block (MINT_FETCH_LDS): streams the own
@@ -1179,18 +1393,21 @@ template <int DT, int CPI, int U, int WPB, int R>
 __global__ void __launch_bounds__((WPB + 1) * 64) ring_kernel_lds(const RingArgs a) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     MINT_LDS uint8_t* lds = (MINT_LDS uint8_t*)lds_raw;
+    __shared__ int entry[2];
     if (threadIdx.x < 16) reinterpret_cast<MINT_LDS uint32_t*>(lds)[threadIdx.x] = 0u;
     __syncthreads();
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     const bool fetcher = wib == WPB;
-    const Seat st = take_seat(a, WPB, fetcher ? 0 : wib);
+    const Seat st = take_seat(a, WPB, fetcher ? 0 : wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
     const Role role = role_of(a, st.p, st.h);
     if (fetcher) {
         if (role.load) row_fetcher<U, WPB, R>(a, st, role, lds);
         return;
     }
-    walk_as<PROTO_LL128, DT, CPI, U, true>(a, st, role, lds_port(lds, wib, a.fetch_depth, U));
+    if (role.save && !seats_confirmed(a, st.sequence)) return;
+    walk_as<PROTO_LL128, DT, CPI, U, true>(a, st.p, st.h, st.w, role,
+                                           lds_port(lds, wib, a.fetch_depth, U));
 }
 
 }  // namespace mint

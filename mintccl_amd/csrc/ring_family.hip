@@ -36,6 +36,30 @@ int resident_blocks_per_cu(Kernel kernel, int threads, size_t lds_bytes) {
     return per_cu < 1 ? 1 : per_cu;
 }
 
+// Blocks of `kernel` the current device holds at once.  The occupancy of a
+// kernel at a block size does not change, so it is asked once - per device: a
+// process may drive several, and they need not be alike.  `memo` holds one
+// entry per device (0 = not asked yet).  Negative on failure.
+constexpr int kMemoDevices = 64;
+template <typename Kernel>
+int resident_capacity(Kernel kernel, int threads, size_t lds_bytes, std::atomic<int>* memo) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMemoDevices) return -1;
+    int per_cu = memo[dev].load(std::memory_order_relaxed);
+    if (per_cu == 0) {
+        per_cu = resident_blocks_per_cu(kernel, threads, lds_bytes);
+        if (per_cu < 0) return -1;
+        memo[dev].store(per_cu, std::memory_order_relaxed);
+    }
+    static std::atomic<int> cus[kMemoDevices] = {};
+    int ncu = cus[dev].load(std::memory_order_relaxed);
+    if (ncu == 0) {
+        ncu = device_cus();
+        cus[dev].store(ncu, std::memory_order_relaxed);
+    }
+    return per_cu * ncu;
+}
+
 // Launch a plan whose grid fits `capacity` blocks.  Compute units set apart for
 // origins need a larger grid (blocks with nothing to do fill the rounds): where
 // that one does not fit and the plain one does, the plain order runs.
@@ -70,18 +94,11 @@ int launch_ring_lds(const Plan& plan, hipStream_t stream) {
         const int threads = plan.threads + 64;
         const size_t lds_bytes = kLdsHeader + (size_t)wpb * plan.args.fetch_depth *
                                                   (size_t)plan.unroll * kBlockMsg;
-        static std::atomic<int> cached[2][2] = {};       // [wpb == 7][unroll == 2]
-        static std::atomic<int> cus{0};
-        std::atomic<int>& memo = cached[wpb == 7][plan.unroll == 2];
-        int per_cu = memo.load(std::memory_order_relaxed);
-        if (per_cu == 0) {
-            per_cu = resident_blocks_per_cu(kernel, threads, lds_bytes);
-            if (per_cu < 0) return MINT_ERR_HIP;
-            memo.store(per_cu, std::memory_order_relaxed);
-        }
-        int ncu = cus.load(std::memory_order_relaxed);
-        if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-        if (plan.blocks > per_cu * ncu) return MINT_ERR_RESIDENCY;
+        static std::atomic<int> cached[2][2][kMemoDevices] = {};   // [wpb == 7][unroll == 2][device]
+        const int capacity = resident_capacity(kernel, threads, lds_bytes,
+                                               cached[wpb == 7][plan.unroll == 2]);
+        if (capacity < 0) return MINT_ERR_HIP;
+        if (plan.blocks > capacity) return MINT_ERR_RESIDENCY;
         hipLaunchKernelGGL(kernel, dim3((unsigned)plan.blocks), dim3((unsigned)threads), lds_bytes,
                            stream, plan.args);
         return launch_status();
@@ -97,22 +114,13 @@ int launch_ring_u(const Plan& plan, hipStream_t stream) {
         case 2: kernel = ring_kernel<PROTO, DT, CP, 2>; break;
         default: kernel = ring_kernel<PROTO, DT, CP, 1>; break;
     }
-    // The occupancy of a kernel at a block size does not change: ask once
-    // (per block size) and keep it.  (These statics are per template
-    // instantiation, i.e. per kernel family.)
-    static std::atomic<int> cached[3][9] = {};       // [unroll][threads / 64]
-    static std::atomic<int> cus{0};
-    std::atomic<int>& memo = cached[plan.unroll == 4 ? 2 : (plan.unroll == 2 ? 1 : 0)]
-                                   [plan.threads / 64];
-    int per_cu = memo.load(std::memory_order_relaxed);
-    if (per_cu == 0) {
-        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
-        if (per_cu < 0) return MINT_ERR_HIP;
-        memo.store(per_cu, std::memory_order_relaxed);
-    }
-    int ncu = cus.load(std::memory_order_relaxed);
-    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    return launch_resident(kernel, plan, per_cu * ncu, stream);
+    // (These statics are per template instantiation, i.e. per kernel family.)
+    static std::atomic<int> cached[3][9][kMemoDevices] = {};   // [unroll][threads / 64][device]
+    const int capacity = resident_capacity(
+        kernel, plan.threads, 0,
+        cached[plan.unroll == 4 ? 2 : (plan.unroll == 2 ? 1 : 0)][plan.threads / 64]);
+    if (capacity < 0) return MINT_ERR_HIP;
+    return launch_resident(kernel, plan, capacity, stream);
 }
 
 template <int PROTO, int DT>
@@ -129,18 +137,10 @@ int launch_ring_cp(const Plan& plan, int cache_policy, hipStream_t stream) {
 template <int DT, int CP>
 int launch_tree(const Plan& plan, hipStream_t stream) {
     void (*kernel)(const RingArgs) = tree_kernel<DT, CP>;
-    static std::atomic<int> cached[9] = {};          // [threads / 64]
-    static std::atomic<int> cus{0};
-    std::atomic<int>& memo = cached[plan.threads / 64];
-    int per_cu = memo.load(std::memory_order_relaxed);
-    if (per_cu == 0) {
-        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
-        if (per_cu < 0) return MINT_ERR_HIP;
-        memo.store(per_cu, std::memory_order_relaxed);
-    }
-    int ncu = cus.load(std::memory_order_relaxed);
-    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    return launch_resident(kernel, plan, per_cu * ncu, stream);
+    static std::atomic<int> cached[9][kMemoDevices] = {};      // [threads / 64][device]
+    const int capacity = resident_capacity(kernel, plan.threads, 0, cached[plan.threads / 64]);
+    if (capacity < 0) return MINT_ERR_HIP;
+    return launch_resident(kernel, plan, capacity, stream);
 }
 
 // Allgather, temporal schedule (LL128, bytes): one wavefront per (rank,
@@ -148,18 +148,10 @@ int launch_tree(const Plan& plan, hipStream_t stream) {
 template <int CP>
 int launch_temporal(const Plan& plan, hipStream_t stream) {
     void (*kernel)(const RingArgs) = temporal_kernel<CP>;
-    static std::atomic<int> cached[9] = {};          // [threads / 64]
-    static std::atomic<int> cus{0};
-    std::atomic<int>& memo = cached[plan.threads / 64];
-    int per_cu = memo.load(std::memory_order_relaxed);
-    if (per_cu == 0) {
-        per_cu = resident_blocks_per_cu(kernel, plan.threads, 0);
-        if (per_cu < 0) return MINT_ERR_HIP;
-        memo.store(per_cu, std::memory_order_relaxed);
-    }
-    int ncu = cus.load(std::memory_order_relaxed);
-    if (ncu == 0) { ncu = device_cus(); cus.store(ncu, std::memory_order_relaxed); }
-    return launch_resident(kernel, plan, per_cu * ncu, stream);
+    static std::atomic<int> cached[9][kMemoDevices] = {};      // [threads / 64][device]
+    const int capacity = resident_capacity(kernel, plan.threads, 0, cached[plan.threads / 64]);
+    if (capacity < 0) return MINT_ERR_HIP;
+    return launch_resident(kernel, plan, capacity, stream);
 }
 
 template <int DT>

@@ -43,10 +43,7 @@ __device__ __forceinline__ void temporal_walk(const RingArgs& a, const int h, co
     const uint32_t W = (uint32_t)a.waves, K = a.k_per_wave;
     const uint32_t chan = a.credit_off + (uint32_t)w * kCreditStride;
     const bool origin = h == 0, last = h == n - 1;
-    const uint32_t epoch =
-        a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
-                           as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-                     : a.epoch;
+    const uint32_t epoch = launch_epoch(a);
     const uint64_t flag_hi = (uint64_t)epoch << 32;
 
     uint32_t gs = 0, slot = 0;                  // step counted through the phases, its slot
@@ -287,10 +284,14 @@ __device__ __forceinline__ void temporal_walk(const RingArgs& a, const int h, co
 // Seats are dealt as for the ring kernels.
 template <int CPI>
 __global__ void __launch_bounds__(512) temporal_kernel(const RingArgs a) {
+    __shared__ int entry[2];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
-    const Seat st = take_seat(a, wpb, wib);
+    const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
+    // (every position but the origins' writes the buffers of the ranks it
+    // serves: first make sure every position of the launch has a thread block)
+    if (st.h != 0 && !seats_confirmed(a, st.sequence)) return;
     temporal_walk<CPI>(a, st.h, st.w);
 }
 

@@ -85,11 +85,9 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
     const uint64_t* const out_tail[kTreeArity] = {credit_word(to[0], to_share[0]),
                                                   credit_word(to[1], to_share[1])};
 
-    const uint32_t epoch =
-        a.epoch_word ? __builtin_amdgcn_readfirstlane(__hip_atomic_load(
-                           as_global(a.epoch_word), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-                     : a.epoch;
+    const uint32_t epoch = launch_epoch(a);
     const uint64_t flag_hi = (uint64_t)epoch << 32;
+
     uint32_t credits_seen[kTreeArity] = {0u, 0u};
 
     // Own rows one block ahead (whole blocks only; the ragged last block of a
@@ -256,10 +254,14 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
 // with the local placement a wave-channel's whole tree shares one XCD.
 template <int DT, int CPI>
 __global__ void __launch_bounds__(512) tree_kernel(const RingArgs a) {
+    __shared__ int entry[2];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
-    const Seat st = take_seat(a, wpb, wib);
+    const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
+    // a node that writes a caller's buffer (the root of a reduce, everybody
+    // else in a broadcast) first makes sure every node has a thread block
+    if ((a.op == OP_TREE_REDUCE ? st.h == 0 : st.h != 0) && !seats_confirmed(a, st.sequence)) return;
     tree_walk<DT, CPI>(a, st.h, st.w);
 }
 

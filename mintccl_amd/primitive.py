@@ -61,6 +61,25 @@ def step_mix(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int
                                             iters, what, ptr(sink), _stream(ref)), "mint_step_mix")
 
 
+def step_mix_deep(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int, iters: int,
+                  what: int = 7, ahead: int = 1, partner: bool = True,
+                  sink: torch.Tensor | None = None) -> None:
+    """``step_mix`` with the loads ``ahead`` (1..3) steps ahead of their use and
+    the stores never waited for: ``ahead + 1`` steps in flight per wavefront.
+    ``staging`` holds ``waves * (ahead + 2)`` KiB; ``iters`` is a multiple of
+    ``ahead + 1``; with ``partner`` a wavefront loads the lines another compute
+    unit of its XCD stores."""
+    ref = rows if rows is not None else staging
+    if sink is None and not what & 4:
+        sink = torch.zeros(1, dtype=torch.int32, device=ref.device)
+    nb = lambda t: 0 if t is None else t.numel() * t.element_size()
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(ref.device):
+        _lib.check(_lib.lib().mint_step_mix_deep(ptr(rows), nb(rows), ptr(staging), nb(staging),
+                                                 waves, iters, what, ahead, int(partner), ptr(sink),
+                                                 _stream(ref)), "mint_step_mix_deep")
+
+
 def Sum(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """Elementwise ``rn(a + b)``, one rounding, by the ring kernels' own adder."""
     if a.dtype not in DTYPE_CODE or a.dtype != b.dtype or a.numel() != b.numel():

@@ -58,7 +58,7 @@ def _launch(comm: VirtualComm, s: dict, r: dict, route: list[int] | None,
         # since the launch is asynchronous
         slot = d.slot_bytes
         d.nslots = max(1, -(-packed_bytes(s["count"]) // slot))
-        per_rank = d.nslots * slot + max(4096, slot // 4)
+        per_rank = d.nslots * slot + max(4096, slot // 4) + _lib.TICKET_BYTES
         hops = torch.zeros(comm.world_size * per_rank, dtype=torch.uint8, device=comm.device)
         comm._indirect_staging = hops
         for k in range(comm.world_size):

@@ -33,9 +33,11 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_version_and_strerror():
     L = _lib.lib()
-    assert L.mint_version() >= 100
+    assert L.mint_version() == _lib.VERSION == 102
+    assert L.mint_build_flags() == 0          # the in-tree library is a product build
+    assert _lib.build_flags() == []
     assert L.mint_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert L.mint_strerror(code) not in (b"ok", b"unknown error")
     assert L.mint_strerror(-99) == b"unknown error"
 
@@ -106,8 +108,8 @@ def test_plan_geometry_without_a_gpu():
     d = make_op()
     # 8 pipelines x 9 positions x (16 waves / 4 per block)
     assert L.mint_ring_grid_blocks(d) == 8 * 9 * 4
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256
-    assert L.mint_ring_staging_bytes(make_op(credit_offset=8 << 20)) == (8 << 20) + 8 * 16 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256 + _lib.TICKET_BYTES
+    assert L.mint_ring_staging_bytes(make_op(credit_offset=8 << 20)) == (8 << 20) + 8 * 16 * 256 + _lib.TICKET_BYTES
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER, dtype=_lib.BYTES)) == 8 * 8 * 4
     d = make_op(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
     assert L.mint_ring_grid_blocks(d) == 8 * 32
@@ -116,13 +118,13 @@ def test_plan_geometry_without_a_gpu():
     # allreduce: 8 pipelines x 15 positions, two phases share a slot
     d = make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=16, count_bytes=8 << 20)
     assert L.mint_ring_grid_blocks(d) == 8 * 15 * 4
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 2 * 16 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 2 * 16 * 256 + _lib.TICKET_BYTES
     # alltoall: 64 pipelines x 2 positions; a slot has one share per source rank
     d = make_op(op=_lib.OP_ALLTOALL, dtype=_lib.BYTES, waves_per_channel_group=16)
     for r in range(8):
         d.output[r] = 0x40000000 + r * 0x1000000
     assert L.mint_ring_grid_blocks(d) == 64 * 2 * 4
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 8 * 16 * 256 + _lib.TICKET_BYTES
     d.output[5] = d.input[2] + (3 << 20)                    # an output inside an input
     assert L.mint_ring_grid_blocks(d) == _lib.ERR_ARG
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLREDUCE, waves_per_channel_group=64)) \
@@ -223,10 +225,10 @@ def test_tree_plans_without_a_gpu():
     L = _lib.lib()
     d = make_op(op=_lib.OP_TREE_BROADCAST, dtype=_lib.BYTES, waves_per_channel_group=128, root=3)
     assert L.mint_ring_grid_blocks(d) == 8 * 32
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256 + _lib.TICKET_BYTES
     d = make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=128, root=3)
     assert L.mint_ring_grid_blocks(d) == 8 * 32
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 2 * 128 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 2 * 128 * 256 + _lib.TICKET_BYTES
     # 512 KiB slot / 2 shares = 256 blocks per step
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_TREE_REDUCE, waves_per_channel_group=512)) \
         == _lib.ERR_GEOMETRY
@@ -262,7 +264,7 @@ def test_temporal_allgather_plan_without_a_gpu():
     L = _lib.lib()
     d = make_op(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES, waves_per_channel_group=128)
     assert L.mint_ring_grid_blocks(d) == 8 * 32
-    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256
+    assert L.mint_ring_staging_bytes(d) == (4 << 20) + 128 * 256 + _lib.TICKET_BYTES
     # the same slot takes 8 x 64 blocks of the spatial schedule or 512 of this one
     assert L.mint_ring_grid_blocks(make_op(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES,
                                            waves_per_channel_group=512)) == 8 * 128
@@ -287,7 +289,7 @@ def test_launch_refuses_undersized_staging_before_touching_the_gpu():
     L = _lib.lib()
     d = make_op()
     need = L.mint_ring_staging_bytes(d)
-    assert need == (4 << 20) + 8 * 16 * 256
+    assert need == (4 << 20) + 8 * 16 * 256 + _lib.TICKET_BYTES
     for have in (0, 4 << 20, need - 1):
         d.staging_bytes = have
         assert L.mint_ring_launch(d, None) == _lib.ERR_STAGING

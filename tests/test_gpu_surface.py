@@ -206,12 +206,12 @@ def test_device_epoch_wraps_and_clears(dev):
     seen = []
     for i in range(6):
         if i == 2:
-            comm.epoch_word.fill_(4094)          # two launches before the count starts over
+            comm.epoch_word[0] = 4094            # two launches before the count starts over
         for b, h in zip(bufs, host):
             b.copy_(h)
         comm.run(lambda r: reducescatter(bufs[r], comm))
         comm.check()
-        seen.append(int(comm.epoch_word.item()))
+        seen.append(int(comm.epoch_word[0].item()))
         assert all(np.array_equal(as_bytes(b), w) for b, w in zip(bufs, want)), i
     assert seen == [1, 2, 4095, 1, 2, 3]
 
@@ -348,3 +348,58 @@ def test_captured_collectives_replay(dev):
         comm.check()
         for r in range(world):
             assert torch.equal(a[r], ea[r]) and torch.equal(b[r], eb[r]) and torch.equal(c[r], ec[r]), replay
+
+
+@pytest.mark.gpu
+def test_captured_ll128_launch_replayed_after_an_eager_simple_launch(dev):
+    """A communicator with its epoch in device memory: an LL128 allgather is
+    captured while the launch before it was LL128 too; between the replays an
+    eager Simple broadcast on the same communicator leaves payload in the
+    slots that would pass for sector tags.  The kernel that advances the epoch
+    clears them when the graph runs - the host took no such decision when the
+    graph was captured - so every replay equals the eager result."""
+    from mintccl_amd import _lib
+    from mintccl_amd.allgather import allgather
+    world, n = 8, 52000
+    comm = make_comm(world, device_epoch=True)
+    ins = [torch.zeros(world, n, dtype=torch.float16, device=dev) for _ in range(world)]
+    g = [torch.zeros_like(x) for x in ins]
+
+    def sequence():
+        for r in range(world):
+            g[r].copy_(ins[r])
+        comm.run(lambda r: allgather(g[r], comm))
+
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):
+        sequence()
+    side.synchronize()
+    comm.check()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sequence()
+    n32 = 1 << 18
+    src = torch.arange(n32, dtype=torch.int64)
+    forged = ((((src // 256) % 4095 + 1) << 20) | 1).to(torch.int32)
+    bc = [forged.to(dev) if r == 0 else torch.zeros(n32, dtype=torch.int32, device=dev)
+          for r in range(world)]
+    ptrs = {r: bc[r].data_ptr() for r in range(world)}
+    for replay in range(4):
+        host = [uniform(world * n, -1.0, 1.0, 700 + 10 * replay + r).reshape(world, n)
+                for r in range(world)]
+        for r in range(world):
+            ins[r].copy_(host[r].to(dev))
+        if replay % 2 == 0:
+            d = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n32 * 4, {0: ptrs[0]},
+                             {r: ptrs[r] for r in range(1, world)}, list(range(world)) + [0],
+                             root=0, protocol=_lib.PROTO_SIMPLE)
+            comm.launch(d)
+            comm.check()
+            for t in bc:
+                assert torch.equal(t.cpu(), forged)
+        graph.replay()
+        torch.cuda.synchronize()
+        comm.check()
+        for r in range(world):
+            for c in range(world):
+                assert torch.equal(g[r][c].cpu(), host[c][c]), (replay, r, c)

@@ -89,19 +89,10 @@ def test_static_launch_ll128_after_simple_and_other_geometries(dev, lib):
     is what the next LL128 launch would take for its sector tags, then LL128
     collectives of other shapes on the same array."""
     status = torch.zeros(4, dtype=torch.int64, device=dev)
-    n32 = 3 * 5 * 7 * 1024 + 3
-    # the epoch in the array is unknown here (other tests may have used it):
-    # forge the tags of every epoch the next launch could carry, in turn
-    src = torch.arange(n32, dtype=torch.int64)
-    forged = ((((src // 256) % 4095 + 1) << 20) | 1).to(torch.int32)
-    bufs = [forged.to(dev) if r == 2 else torch.zeros(n32, dtype=torch.int32, device=dev)
-            for r in range(WORLD)]
-    d = descriptor(_lib.OP_BROADCAST, _lib.BYTES, _lib.PROTO_SIMPLE, n32 * 4,
-                   [t.data_ptr() for t in bufs], status, root=2, slot_bytes=64 * 1024, nslots=3)
-    launch_static(lib, d)
+    # (the epoch in the array is unknown here - other tests may have used it -
+    # so the payload forges the tags of every epoch the next launch could carry)
+    forged_simple_broadcast(lib, dev, status)
     assert ok(status)
-    for t in bufs:
-        assert torch.equal(t.cpu(), forged)
     for n, slot, nslots, waves in ((52000, 8 * 32 * 1024, 4, 32), (480, 8 * 1024, 1, 1)):
         host = [uniform(WORLD * n, -1.0, 1.0, 40 + r).reshape(WORLD, n) for r in range(WORLD)]
         g = [h.to(dev) for h in host]
@@ -142,6 +133,105 @@ def test_static_launch_of_the_tree_and_the_temporal_schedule(dev, lib):
     want = ring.allgather([as_bytes(h) for h in host])
     for r in range(WORLD):
         assert np.array_equal(as_bytes(g[r]), want[r]), r
+
+
+def forged_simple_broadcast(lib, dev, status):
+    """A Simple broadcast through the static array whose payload is what an
+    LL128 launch of any epoch would take for its sector tags."""
+    n32 = 3 * 5 * 7 * 1024 + 3
+    src = torch.arange(n32, dtype=torch.int64)
+    forged = ((((src // 256) % 4095 + 1) << 20) | 1).to(torch.int32)
+    bufs = [forged.to(dev) if r == 2 else torch.zeros(n32, dtype=torch.int32, device=dev)
+            for r in range(WORLD)]
+    d = descriptor(_lib.OP_BROADCAST, _lib.BYTES, _lib.PROTO_SIMPLE, n32 * 4,
+                   [t.data_ptr() for t in bufs], status, root=2, slot_bytes=64 * 1024, nslots=3)
+    launch_static(lib, d)
+    for t in bufs:
+        assert torch.equal(t.cpu(), forged)
+
+
+@pytest.mark.gpu
+def test_static_launch_captured_then_replayed_after_a_simple_launch(dev, lib):
+    """An LL128 launch through the static array is captured into a graph while
+    the launch before it was LL128 as well.  Between the replays an eager
+    Simple launch leaves payload in the array that would pass for sector tags:
+    every replay has to clear it by itself (the decision is taken on the
+    device when the graph runs, not on the host when it was captured) and
+    equal the oracle."""
+    status = torch.zeros(4, dtype=torch.int64, device=dev)
+    assert lib.mint_static_init() == _lib.OK
+    n = 52000
+    ins = [torch.zeros(WORLD, n, dtype=torch.float16, device=dev) for _ in range(WORLD)]
+    g = [torch.zeros_like(x) for x in ins]
+    d = descriptor(_lib.OP_ALLGATHER, _lib.BYTES, _lib.PROTO_LL128, n * 2,
+                   [t.data_ptr() for t in g], status, slot_bytes=8 * 32 * 1024, nslots=4, waves=32)
+    for r in range(WORLD):
+        d.staging[r] = 0
+    d.staging_bytes = d.flag_epoch = d.epoch_ptr = d.credit_offset = 0
+    side = torch.cuda.Stream(device=dev)
+
+    def enqueue():
+        for r in range(WORLD):
+            g[r].copy_(ins[r])
+        _lib.check(lib.mint_ring_launch_static(d, side.cuda_stream), "mint_ring_launch_static")
+
+    with torch.cuda.stream(side):
+        enqueue()                                  # LL128 before the capture
+    side.synchronize()
+    assert ok(status)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        enqueue()
+    for replay in range(4):
+        host = [uniform(WORLD * n, -1.0, 1.0, 900 + 10 * replay + r).reshape(WORLD, n)
+                for r in range(WORLD)]
+        for r in range(WORLD):
+            ins[r].copy_(host[r].to(dev))
+        if replay % 2 == 0:
+            forged_simple_broadcast(lib, dev, status)   # eager, between the replays
+            assert ok(status)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ok(status), replay
+        want = ring.allgather([as_bytes(h) for h in host])
+        for r in range(WORLD):
+            assert np.array_equal(as_bytes(g[r]), want[r]), (replay, r)
+
+
+@pytest.mark.gpu
+def test_static_launch_allocates_nothing_and_queues_back_to_back(dev, lib):
+    """A warm call leaves the device's free memory as it was, and two launches
+    queued on one stream with no host synchronisation in between (they share
+    the array, the stream orders them) both equal the oracle."""
+    status = torch.zeros(4, dtype=torch.int64, device=dev)
+    n = 30011
+    hosts, bufs, descs = [], [], []
+    for k in range(2):
+        host = rank_rows(WORLD, n - 1000 * k, "f16", seed0=500 + 20 * k)
+        b = [h.to(dev) for h in host]
+        d = descriptor(_lib.OP_REDUCESCATTER, _lib.F16, _lib.PROTO_LL128, (n - 1000 * k) * 2,
+                       [t.data_ptr() for t in b], status)
+        for r in range(WORLD):
+            d.staging[r] = 0
+        d.staging_bytes = d.flag_epoch = d.epoch_ptr = d.credit_offset = 0
+        hosts.append(host); bufs.append(b); descs.append(d)
+    warm = [h.to(dev) for h in hosts[0]]
+    dw = descriptor(_lib.OP_REDUCESCATTER, _lib.F16, _lib.PROTO_LL128, n * 2,
+                    [t.data_ptr() for t in warm], status)
+    launch_static(lib, dw)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    reserved_before = torch.cuda.memory_reserved(dev)
+    for d in descs:
+        _lib.check(lib.mint_ring_launch_static(d, None), "mint_ring_launch_static")
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert free_after == free_before and torch.cuda.memory_reserved(dev) == reserved_before
+    assert ok(status)
+    for host, b in zip(hosts, bufs):
+        want = ring.reducescatter([as_bytes(h) for h in host], "f16")
+        for r in range(WORLD):
+            assert np.array_equal(as_bytes(b[r]), want[r]), r
 
 
 def test_static_launch_refuses_what_does_not_fit_the_array():
