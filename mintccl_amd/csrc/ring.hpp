@@ -759,6 +759,16 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // follow the sends are then the same number on every path)
     constexpr bool kSendsFirst = PROTO == PROTO_SIMPLE && DT == DT_BYTES && RoleT::send && !LDSF &&
                                  (RoleT::save || !RoleT::recv);
+    // Vector-memory operations such a group issues between its sends and the
+    // wait in front of the step counter, which may stay in flight there (a
+    // wavefront's operations retire in issue order, so waiting until this many
+    // are left is waiting for the sends): U saves of a receiver or U fetches
+    // ahead of an origin - the block under `if (WHOLE && kSendsFirst)` behind
+    // the sends - and, for a receiver, the one store of the credit post under
+    // `if (q.last)`.  Whoever adds or removes an operation there changes this.
+    constexpr int kOpsBehindSends = U + (RoleT::recv ? 1 : 0);
+    static_assert(!kSendsFirst || (RoleT::save != !RoleT::recv),
+                  "a group that sends first either saves (a receiver) or fetches ahead (an origin)");
     auto run_group = [&](auto whole_tag, auto parity_tag) MINT_INLINE_LAMBDA -> bool {
         constexpr bool WHOLE = decltype(whole_tag)::value;
         constexpr int P = decltype(parity_tag)::value;
@@ -914,7 +924,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 // issued after them - a receiver's saves to HBM, an origin's
                 // fetch ahead - and the credit post may stay in flight.
                 if (WHOLE && kSendsFirst)
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(U + (RoleT::recv ? 1 : 0)) : "memory");
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kOpsBehindSends) : "memory");
                 else
                     wait_stores_visible();
                 if (lane_id() == 0) {
