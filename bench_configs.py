@@ -443,16 +443,76 @@ def tree_bench(reps: int, log2s=(10, 14, 17, 20, 23, 26)) -> None:
                  us=round(ms * 1e3, 2), hbm_bytes=world * nbytes, ok=ok, grid=comm.last_grid)
 
 
+def hypercube_bench(reps: int, log2s=(14, 20, 26)) -> None:
+    """Reduce-scatter and allgather over the hypercube (3 exchanges for 8
+    ranks) beside the ring (7 hops), 8 ranks, 16 KiB to 64 MiB per rank,
+    launched from prepared descriptors; the reduce-scatter is checked against
+    the device adder folded in the hypercube's / the ring's order, the
+    allgather against the rows it gathers."""
+    from mintccl_amd import hypercube, primitive
+    world = 8
+    comm = comm_for(world, 0)
+    ring = list(range(world)) + [0]
+    for log2 in log2s:
+        nbytes = 1 << log2
+        row = nbytes // world
+        n = row // 2
+        g = torch.Generator(device=DEV).manual_seed(10)
+        src = [(torch.rand(world, n, generator=g, device=DEV) * 2 - 1).to(torch.float16)
+               for _ in range(world)]
+
+        def cube_sum(tree, r: int) -> torch.Tensor:
+            if isinstance(tree, int):
+                return src[tree][r].clone()
+            return primitive.Sum(cube_sum(tree[0], r), cube_sum(tree[1], r))
+
+        want = {"hypercube": [cube_sum(hypercube.order(world, r), r) for r in range(world)],
+                "ring": [fold_device([x[r] for x in src], [(r + i) % world for i in range(world)])
+                         for r in range(world)]}
+        bufs = [x.clone() for x in src]
+        ptrs = {r: bufs[r].data_ptr() for r in range(world)}
+        for topo, rs, ag in (("ring", _lib.OP_REDUCESCATTER, _lib.OP_ALLGATHER),
+                             ("hypercube", _lib.OP_HYPERCUBE_REDUCESCATTER,
+                              _lib.OP_HYPERCUBE_ALLGATHER)):
+            for b, x in zip(bufs, src):
+                b.copy_(x)
+            d = comm.make_op(rs, _lib.F16, row, ptrs, ptrs, ring, row_stride=row,
+                             protocol=_lib.PROTO_LL128)
+            comm.launch(d)
+            comm.check()
+            ok = all(torch.equal(bufs[r][r], want[topo][r]) for r in range(world))
+            # (timed launches keep adding into row r of rank r: the values no longer matter)
+            ms = time_ms(lambda: comm.launch(d), reps * 4)
+            comm.check()
+            emit(config="hypercube", op="reducescatter", topology=topo, world=world, bytes=nbytes,
+                 us=round(ms * 1e3, 2), hbm_bytes=(world + 1) * nbytes, ok=ok, grid=comm.last_grid)
+            for r, b in enumerate(bufs):
+                b.zero_()
+                b[r].copy_(src[r][r])
+            d = comm.make_op(ag, _lib.BYTES, row, ptrs, ptrs, ring, row_stride=row,
+                             protocol=_lib.PROTO_LL128)
+            comm.launch(d)
+            comm.check()
+            ok = all(torch.equal(b[c], src[c][c]) for b in bufs for c in range(world))
+            ms = time_ms(lambda: comm.launch(d), reps * 4)
+            comm.check()
+            emit(config="hypercube", op="allgather", topology=topo, world=world, bytes=nbytes,
+                 us=round(ms * 1e3, 2), hbm_bytes=world * nbytes, ok=ok, grid=comm.last_grid)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--staging", choices=("both", "reference", "tuned"), default="both")
     ap.add_argument("--quick", action="store_true", help="fewer repetitions, sweep to 16 MiB")
     ap.add_argument("--only", type=int, default=0,
-                    help="run one config (1..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring)")
+                    help="run one config (1..5; 8 = allreduce; 9 = alltoall; 10 = tree against ring; "
+                         "11 = hypercube against ring)")
     ap.add_argument("--shard-log2", default="",
                     help="config 5: only these shard sizes (log2 of bytes, comma separated)")
     ap.add_argument("--tree-log2", default="10,14,17,20,23,26",
                     help="config 10: log2 of the message sizes (bytes per rank)")
+    ap.add_argument("--cube-log2", default="14,17,20,23,26",
+                    help="config 11: log2 of the message sizes (bytes per rank)")
     args = ap.parse_args()
     global STAGING
     STAGING = ("reference", "tuned") if args.staging == "both" else (args.staging,)
@@ -475,6 +535,8 @@ def main() -> int:
         alltoall_bench(reps)
     if args.only in (0, 10):
         tree_bench(reps, tuple(int(x) for x in args.tree_log2.split(",")))
+    if args.only in (0, 11):
+        hypercube_bench(reps, tuple(int(x) for x in args.cube_log2.split(",")))
     return 0
 
 

@@ -77,6 +77,19 @@ typedef enum {
                                   rounding per addition.  LL128 only.  slot_bytes
                                   of a TREE_REDUCE holds two shares (one per
                                   child). */
+    MINT_OP_HYPERCUBE_REDUCESCATTER = 10, /* reduce-scatter and allgather over a */
+    MINT_OP_HYPERCUBE_ALLGATHER = 11,     /* hypercube, the last open topology of the
+                                  reference's roadmap (README.md:52-55): recursive
+                                  halving / doubling, log2(world) exchanges instead
+                                  of world - 1 hops; world is 2, 4 or 8.  Node i is
+                                  rank ring[i]; in exchange k = 0.. nodes i and
+                                  i ^ (world >> (k + 1)) split the rows they still
+                                  hold.  Buffers as for REDUCESCATTER / ALLGATHER;
+                                  the value a node passes on is
+                                  ((own + partner 0) + partner 1) + partner 2, one
+                                  rounding per addition.  LL128 only.  slot_bytes
+                                  holds world - 1 shares (the streams a rank
+                                  receives). */
     MINT_OP_ALLGATHER_TEMPORAL = 9 /* 6_allgather.py:25-77, the schedule the
                                   reference's allgather launches (:157): the whole
                                   grid moves rank 0's row round the ring, then rank
@@ -148,9 +161,9 @@ typedef struct {
                               words sit behind the slots, outside a buffer
                               that only holds nslots * slot_bytes) */
     uint64_t count_bytes;  /* SENDRECV/BROADCAST/REDUCE/ALLREDUCE/TREE_*: bytes of the
-                              buffer; ALLGATHER(_TEMPORAL)/REDUCESCATTER/ALLTOALL: bytes of
-                              one row */
-    uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER/ALLTOALL: bytes between rows */
+                              buffer; ALLGATHER(_TEMPORAL)/REDUCESCATTER/ALLTOALL/HYPERCUBE_*:
+                              bytes of one row */
+    uint64_t row_stride;   /* ALLGATHER/REDUCESCATTER/ALLTOALL/HYPERCUBE_*: bytes between rows */
     uint32_t slot_bytes;   /* staging bytes of one step over all pipelines;
                               multiple of 1024, >= 1024 per pipeline (per
                               pipeline and phase for ALLREDUCE, which has 2;

@@ -33,7 +33,8 @@ LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
 F16, BF16, F32, BYTES = 0, 1, 2, 3
 PROTO_LL128, PROTO_SIMPLE = 0, 1
 (OP_SENDRECV, OP_BROADCAST, OP_REDUCE, OP_ALLGATHER, OP_REDUCESCATTER, OP_ALLREDUCE,
- OP_ALLTOALL, OP_TREE_BROADCAST, OP_TREE_REDUCE, OP_ALLGATHER_TEMPORAL) = range(10)
+ OP_ALLTOALL, OP_TREE_BROADCAST, OP_TREE_REDUCE, OP_ALLGATHER_TEMPORAL,
+ OP_HYPERCUBE_REDUCESCATTER, OP_HYPERCUBE_ALLGATHER) = range(12)
 PLACE_SPREAD, PLACE_LOCAL = 0, 1
 FETCH_INLINE, FETCH_LDS = 0, 1
 

@@ -7,7 +7,8 @@ its own share of the staging - the default here, it is the faster one.
 *Temporal* (``:25-77``, the one the reference's host function launches): the
 whole grid moves rank 0's row round the ring, then rank 1's, and so on,
 through staging for one row - ``schedule="temporal"`` or
-``MINTCCL_ALLGATHER=temporal`` (LL128 only)."""
+``MINTCCL_ALLGATHER=temporal`` (LL128 only).  ``MINTCCL_TOPOLOGY=hypercube``
+doubles recursively over a hypercube instead (``mintccl_amd.hypercube``)."""
 from __future__ import annotations
 
 import os
@@ -21,6 +22,9 @@ from .common import VirtualComm
 
 def allgather(buff: torch.Tensor, comm: VirtualComm | None = None,
               schedule: str | None = None) -> None:
+    from . import hypercube, tree
+    if schedule is None and tree.topology_env() == "hypercube":
+        return hypercube.allgather(buff, comm)
     if schedule is None:
         schedule = os.getenv("MINTCCL_ALLGATHER", "spatial").lower()
     if schedule not in ("spatial", "temporal"):

@@ -185,6 +185,13 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         granule = wpb * 8
         waves = max(granule, min(TUNED_SLOT_BLOCKS, TUNED_TOTAL_WAVES // world) // granule * granule)
         return fit(shares, max_nslots, waves, granule)
+    if op in (_lib.OP_HYPERCUBE_REDUCESCATTER, _lib.OP_HYPERCUBE_ALLGATHER):
+        # world rows x world nodes, one wavefront per (row, node, wave-channel);
+        # a rank's slot has a share per stream it receives: world - 1
+        granule = wpb
+        waves = max(granule, min(TUNED_SLOT_BUDGET // 1024 // max(1, world - 1),
+                                 TUNED_TOTAL_WAVES // (world * world)) // granule * granule)
+        return fit(max(1, world - 1), max_nslots, waves, granule)
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
     real_pipes = pipes
     if op == _lib.OP_ALLREDUCE:
@@ -442,6 +449,9 @@ class VirtualComm:
         tree = op in (_lib.OP_TREE_BROADCAST, _lib.OP_TREE_REDUCE)
         if op == _lib.OP_TREE_REDUCE:
             pipes = 2             # a slot has a share per child
+        hyper = op in (_lib.OP_HYPERCUBE_REDUCESCATTER, _lib.OP_HYPERCUBE_ALLGATHER)
+        if hyper:
+            pipes = max(1, self.world_size - 1)   # ... per stream a rank receives
         threads = self.threads_per_block
         reducing = op in (_lib.OP_REDUCE, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE)
         if self.auto_geometry:
@@ -465,7 +475,8 @@ class VirtualComm:
                     "slot size must be a multiple of 1 KiB, at least 1 KiB per pipeline")
             # (an alltoall has twice `pipes` groups of wave-channels per rank: it
             # sends `world` rows and receives `world` rows)
-            groups = 2 * pipes if op == _lib.OP_ALLTOALL else (1 if tree else pipes)
+            groups = 2 * pipes if op == _lib.OP_ALLTOALL else (
+                1 if tree else (self.world_size if hyper else pipes))
             d.waves_per_channel_group = _largest_divisor_at_most(
                 step_blocks, max(1, self.waves_per_rank // groups))
         d.threads_per_block = threads
@@ -480,6 +491,8 @@ class VirtualComm:
                 real_pipes = self.world_size * self.world_size
             if tree:
                 real_pipes = 1
+            if hyper:
+                real_pipes = self.world_size
             channels = real_pipes * -(-d.waves_per_channel_group // wpb)
             if channels % 8:
                 d.placement = _lib.PLACE_SPREAD

@@ -7,6 +7,7 @@
 
 #include "kernels.hpp"
 #include "ring_launch.hpp"
+#include "hypercube.hpp"
 #include "temporal.hpp"
 #include "tree.hpp"
 
@@ -47,11 +48,16 @@ inline bool aligned16(const void* p) { return aligned16(reinterpret_cast<uint64_
 
 bool reducing(int op) {
     return op == MINT_OP_REDUCE || op == MINT_OP_REDUCESCATTER || op == MINT_OP_ALLREDUCE ||
-           op == MINT_OP_TREE_REDUCE;
+           op == MINT_OP_TREE_REDUCE || op == MINT_OP_HYPERCUBE_REDUCESCATTER;
+}
+bool over_hypercube(int op) {
+    return op == MINT_OP_HYPERCUBE_REDUCESCATTER || op == MINT_OP_HYPERCUBE_ALLGATHER;
 }
 bool over_tree(int op) { return op == MINT_OP_TREE_BROADCAST || op == MINT_OP_TREE_REDUCE; }
 static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE == OP_TREE_REDUCE &&
-                  MINT_OP_ALLGATHER_TEMPORAL == OP_ALLGATHER_TEMPORAL,
+                  MINT_OP_ALLGATHER_TEMPORAL == OP_ALLGATHER_TEMPORAL &&
+                  MINT_OP_HYPERCUBE_REDUCESCATTER == OP_HYPER_REDUCESCATTER &&
+                  MINT_OP_HYPERCUBE_ALLGATHER == OP_HYPER_ALLGATHER,
               "op codes");
 
 // Everything the launch derives from the descriptor.  `for_launch`: also
@@ -60,12 +66,16 @@ static_assert(MINT_OP_TREE_BROADCAST == OP_TREE_BROADCAST && MINT_OP_TREE_REDUCE
 int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
               const mint_ring_debug* dbg = nullptr) {
     if (!op || !plan) return MINT_ERR_ARG;
-    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_ALLGATHER_TEMPORAL) return MINT_ERR_ARG;
+    if (op->op < MINT_OP_SENDRECV || op->op > MINT_OP_HYPERCUBE_ALLGATHER) return MINT_ERR_ARG;
     if (op->protocol != MINT_PROTO_LL128 && op->protocol != MINT_PROTO_SIMPLE) return MINT_ERR_ARG;
     if (op->world < 1 || op->world > MINT_MAX_RANKS) return MINT_ERR_ARG;
     // the tree kernels and the temporal allgather speak LL128 only
     const bool temporal = op->op == MINT_OP_ALLGATHER_TEMPORAL;
-    if ((over_tree(op->op) || temporal) && op->protocol != MINT_PROTO_LL128) return MINT_ERR_ARG;
+    const bool hyper = over_hypercube(op->op);
+    if ((over_tree(op->op) || temporal || hyper) && op->protocol != MINT_PROTO_LL128)
+        return MINT_ERR_ARG;
+    // a hypercube has 2^d corners
+    if (hyper && (op->world & (op->world - 1))) return MINT_ERR_ARG;
     if (op->dtype < MINT_F16 || op->dtype > MINT_BYTES) return MINT_ERR_ARG;
     if (reducing(op->op) && op->dtype == MINT_BYTES) return MINT_ERR_ARG;
     if (op->cache_policy < 0 || op->cache_policy > 2) return MINT_ERR_ARG;
@@ -91,7 +101,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     const bool allreduce = op->op == MINT_OP_ALLREDUCE;
     const bool alltoall = op->op == MINT_OP_ALLTOALL;
     const bool rowwise = op->op == MINT_OP_ALLGATHER || op->op == MINT_OP_REDUCESCATTER ||
-                         allreduce || alltoall || temporal;
+                         allreduce || alltoall || temporal || hyper;
     // (the temporal allgather moves its `world` rows one after the other
     // through one pipeline)
     a.pipes = alltoall ? op->world * op->world : (rowwise && !temporal ? op->world : 1);
@@ -101,6 +111,8 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
     a.shares = alltoall ? op->world : a.pipes * a.phases;
     // a node of a reducing tree receives from two children: a share of its slots each
     if (op->op == MINT_OP_TREE_REDUCE) a.shares = kTreeArity;
+    // a corner of a hypercube receives world - 1 streams (hypercube.hpp)
+    if (hyper) a.shares = op->world > 1 ? op->world - 1 : 1;
 
     // ring / route
     bool seen[MINT_MAX_RANKS] = {};
@@ -137,7 +149,7 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         }
         case MINT_OP_ALLTOALL: a.hops = 1; break;
         default:
-            a.hops = op->op == MINT_OP_ALLGATHER || temporal ? op->world - 1
+            a.hops = op->op == MINT_OP_ALLGATHER || temporal || hyper ? op->world - 1
                      : allreduce                             ? 2 * op->world - 2
                                                              : op->world;
             for (int p = 0; p < op->world; ++p) a.start[p] = (uint8_t)index_of(p);
@@ -178,13 +190,13 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         if (receives && (!op->staging[rank] || !aligned16(op->staging[rank])))
             return op->staging[rank] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
     }
-    for (int r = 0; r < op->world && temporal && !plan->empty; ++r) {
+    for (int r = 0; r < op->world && (temporal || hyper) && !plan->empty; ++r) {
         // every rank is origin once and receiver world - 1 times
         if (!op->input[r] || !op->output[r]) return MINT_ERR_ARG;
         if (!op->staging[r] || !aligned16(op->staging[r]))
             return op->staging[r] ? MINT_ERR_ALIGN : MINT_ERR_ARG;
     }
-    for (int p = 0; p < a.pipes && !plan->empty && !over_tree(op->op) && !temporal; ++p) {
+    for (int p = 0; p < a.pipes && !plan->empty && !over_tree(op->op) && !temporal && !hyper; ++p) {
         for (int h = 0; h <= a.hops; ++h) {
             const int rank = alltoall ? (h == 0 ? p / op->world : p % op->world)
                                       : a.cyc[(a.start[p] + h) % a.cyc_len];
@@ -682,7 +694,7 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
     const int err = make_plan(op, &plan);
     if (err != MINT_OK) return err;
     if (plan.empty) return MINT_OK;
-    if (over_tree(op->op) || op->op == MINT_OP_ALLGATHER_TEMPORAL)
+    if (over_tree(op->op) || over_hypercube(op->op) || op->op == MINT_OP_ALLGATHER_TEMPORAL)
         return MINT_ERR_ARG;                        // listed for the ring walks only
     const RingArgs& a = plan.args;
     if (pipeline < 0 || pipeline >= a.pipes || position < 0 || position > a.hops || wave < 0 ||

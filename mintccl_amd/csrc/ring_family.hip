@@ -2,6 +2,7 @@
 // 3 bytes) and their launcher.
 #include <atomic>
 
+#include "hypercube.hpp"
 #include "ring_launch.hpp"
 #include "temporal.hpp"
 #include "tree.hpp"
@@ -143,6 +144,17 @@ int launch_tree(const Plan& plan, hipStream_t stream) {
     return launch_resident(kernel, plan, capacity, stream);
 }
 
+// Reduce-scatter / allgather over a hypercube (LL128): one wavefront per (row,
+// node, wave-channel), all of them resident like a ring's.
+template <int DT, int CP>
+int launch_hyper(const Plan& plan, hipStream_t stream) {
+    void (*kernel)(const RingArgs) = hyper_kernel<DT, CP>;
+    static std::atomic<int> cached[9][kMemoDevices] = {};      // [threads / 64][device]
+    const int capacity = resident_capacity(kernel, plan.threads, 0, cached[plan.threads / 64]);
+    if (capacity < 0) return MINT_ERR_HIP;
+    return launch_resident(kernel, plan, capacity, stream);
+}
+
 // Allgather, temporal schedule (LL128, bytes): one wavefront per (rank,
 // wave-channel).
 template <int CP>
@@ -165,6 +177,13 @@ int launch_family(const Plan& plan, int protocol, int cache_policy, hipStream_t 
             }
         } else {
             return MINT_ERR_ARG;
+        }
+    }
+    if (plan.args.op == OP_HYPER_REDUCESCATTER || plan.args.op == OP_HYPER_ALLGATHER) {
+        switch (cache_policy) {
+            case 0: return launch_hyper<DT, 0>(plan, stream);
+            case 1: return launch_hyper<DT, 1>(plan, stream);
+            default: return launch_hyper<DT, 2>(plan, stream);
         }
     }
     if (plan.args.op == OP_TREE_BROADCAST || plan.args.op == OP_TREE_REDUCE) {

@@ -1,6 +1,8 @@
 """Ring reduce-scatter (``7_reducescatter.py``): ``buff`` is ``(world, n)``;
 after the call row r of rank r holds the sum over ranks of their row r,
-accumulated in ring order starting from rank r's own value."""
+accumulated in ring order starting from rank r's own value.
+``MINTCCL_TOPOLOGY=hypercube`` halves recursively instead
+(``mintccl_amd.hypercube``)."""
 from __future__ import annotations
 
 import torch
@@ -12,6 +14,9 @@ from .common import VirtualComm
 
 
 def reducescatter(buff: torch.Tensor, comm: VirtualComm | None = None) -> None:
+    from . import hypercube, tree
+    if tree.topology_env() == "hypercube":
+        return hypercube.reducescatter(buff, comm)
     comm = comm_or_default(comm)
     check_buffer(buff, comm)
     if buff.numel() % comm.world_size:

@@ -189,12 +189,16 @@ def reducescatter() -> bool:
     _run_all(comm, lambda r: op(bufs[r], comm))
     if inputs is None:
         return True
+    from . import hypercube, tree
     ring, ok = ring_of(comm), True
+    cube = tree.topology_env() == "hypercube"   # the operator halved recursively
     for r in range(world):
         rows = [x[r] for x in inputs]
         if r == 0:
             _order_free_distance(r, bufs[r][r], rows)
-        ok &= _report(r, bufs[r][r], _ring_fold(rows, ring, r), r == 0)
+        want = (_cube_fold(rows, hypercube.nodes(ring), r) if cube
+                else _ring_fold(rows, ring, r))
+        ok &= _report(r, bufs[r][r], want, r == 0)
     return ok
 
 
@@ -246,6 +250,57 @@ def _tree_fold(rows: list[torch.Tensor], order: list[int], h: int = 0) -> torch.
     return acc
 
 
+def _cube_fold(rows: list[torch.Tensor], order: list[int], rank: int) -> torch.Tensor:
+    """Row of ``rank`` after recursive halving over the cube whose corner i is
+    ``order[i]``: the nested additions ``hypercube.order`` names."""
+    from . import hypercube
+
+    def fold(tree):
+        if isinstance(tree, int):
+            return rows[order[tree]].clone()
+        return fold(tree[0]) + fold(tree[1])
+    return fold(hypercube.order(len(order), order.index(rank)))
+
+
+def hypercube_reducescatter() -> bool:
+    """What 7_reducescatter.py:100-116 checks, over a hypercube (README.md:52-55)."""
+    from ._ops import ring_of
+    from .hypercube import nodes, reducescatter as op
+    comm = VirtualComm()
+    world = comm.world_size
+    bufs = _reduction_inputs(comm, (world, common.test_count() // world))
+    inputs = [b.clone() for b in bufs] if common.test_mode() else None
+    _run_all(comm, lambda r: op(bufs[r], comm))
+    if inputs is None:
+        return True
+    order, ok = nodes(ring_of(comm)), True
+    for r in range(world):
+        rows = [x[r] for x in inputs]
+        if r == 0:
+            _order_free_distance(r, bufs[r][r], rows)
+        ok &= _report(r, bufs[r][r], _cube_fold(rows, order, r), r == 0)
+    return ok
+
+
+def hypercube_allgather() -> bool:
+    """What 6_allgather.py:160-178 checks, over a hypercube (README.md:52-55)."""
+    from .hypercube import allgather as op
+    comm = VirtualComm()
+    dev, world = comm.device, comm.world_size
+    n = common.test_count() // world
+    g = _gen(dev)
+    bufs = []
+    for r in range(world):
+        b = torch.zeros(world, n, device=dev)
+        b[r].random_(generator=g)
+        bufs.append(b)
+    want = torch.stack([bufs[r][r] for r in range(world)])
+    _run_all(comm, lambda r: op(bufs[r], comm))
+    if not common.test_mode():
+        return True
+    return all([_report(r, bufs[r], want, r == 0) for r in range(world)])
+
+
 def tree_broadcast() -> bool:
     """What 4_broadcast.py:104-126 checks, down the binary tree (README.md:52-55)."""
     from .tree import broadcast as op
@@ -285,8 +340,13 @@ def main(name: str) -> int:
              "sendrecv_buffer": lambda: sendrecv(sendrecv_buffer),
              "broadcast": broadcast, "reduce": reduce, "allgather": allgather,
              "reducescatter": reducescatter, "allreduce": allreduce, "alltoall": alltoall,
-             "tree_broadcast": tree_broadcast, "tree_reduce": tree_reduce}
+             "tree_broadcast": tree_broadcast, "tree_reduce": tree_reduce,
+             "hypercube_reducescatter": hypercube_reducescatter,
+             "hypercube_allgather": hypercube_allgather}
     if name == "all":
+        world = common.world_size_env()
+        if world & (world - 1):         # no hypercube over this many ranks
+            tests = {k: fn for k, fn in tests.items() if not k.startswith("hypercube")}
         return 0 if all([fn() for fn in tests.values()]) else 1
     return 0 if tests[name]() else 1
 

@@ -222,6 +222,73 @@ def tree_reduce(xs: list, root: int, dtype: str, ring: list[int] | None = None) 
     return out
 
 
+def hypercube_nodes(ring: list[int]) -> list[int]:
+    """Ranks in corner order of the hypercube laid over the ring: corner i is
+    the i-th rank of the ring."""
+    return list(ring[:-1])
+
+
+def hypercube_reducescatter(xs: list, dtype: str, ring: list[int] | None = None) -> list:
+    """Reduce-scatter by recursive halving ("Hypercube" is an open item of the
+    reference's roadmap, ``README.md:52-55``; the reference holds no code for
+    it, so the order of the additions is this build's definition - parity with
+    the reference is unpinned by construction).  xs[r] = rank r's (N, n) buffer
+    as bytes, N = 2^d.  Played as the exchanges themselves: every corner starts
+    with its own values of all N rows; in exchange k = 0 .. d-1 corner i and
+    corner i ^ D, D = N >> (k + 1), split the rows both still hold - a row of
+    corner c stays with the one of the two whose bit D equals c's - and the
+    keeper's partial sum becomes keeper's + partner's, one rounding
+    (``comp_ll128``, ``protocol.py:142-156``).  After d exchanges corner i holds
+    row i of its rank.  Buffers as ``reducescatter``: only row r of rank r
+    changes.  Pinned: against hand-computed values that tell this order from
+    the ring's and from the binary tree's; equal to ``reducescatter`` for
+    N = 2; within (N - 1) half-ulp steps of the exact sum."""
+    n_ranks = len(xs)
+    if n_ranks < 1 or n_ranks & (n_ranks - 1):
+        raise ValueError("a hypercube has 2^d corners")
+    ring = ring or identity_ring(n_ranks)
+    corners = hypercube_nodes(ring)
+    rows = [_bytes(x).reshape(n_ranks, -1) for x in xs]
+    # held[i][c]: corner i's partial sum of the row that belongs to corner c
+    held = [{c: rows[corners[i]][corners[c]].copy() for c in range(n_ranks)}
+            for i in range(n_ranks)]
+    span = n_ranks >> 1
+    while span:
+        after = []
+        for i in range(n_ranks):
+            partner = i ^ span
+            after.append({c: add_rn(held[i][c], held[partner][c], dtype)
+                          for c in held[i] if (c & span) == (i & span)})
+        held, span = after, span >> 1
+    out = [r.copy() for r in rows]
+    for i in range(n_ranks):
+        assert list(held[i]) == [i]
+        out[corners[i]][corners[i]] = held[i][i]
+    return [o.reshape(-1) for o in out]
+
+
+def hypercube_allgather(xs: list, ring: list[int] | None = None) -> list:
+    """Allgather by recursive doubling: the exchanges of
+    ``hypercube_reducescatter`` backwards, every corner handing its partner all
+    rows it holds.  Bytes only move, so the result is ``allgather``'s; played
+    out to check that the exchanges reach every corner."""
+    n_ranks = len(xs)
+    if n_ranks < 1 or n_ranks & (n_ranks - 1):
+        raise ValueError("a hypercube has 2^d corners")
+    corners = hypercube_nodes(ring or identity_ring(n_ranks))
+    rows = [_bytes(x).reshape(n_ranks, -1) for x in xs]
+    held = [{i: rows[corners[i]][corners[i]]} for i in range(n_ranks)]
+    span = 1
+    while span < n_ranks:
+        held = [{**held[i], **held[i ^ span]} for i in range(n_ranks)]
+        span <<= 1
+    out = [r.copy() for r in rows]
+    for i in range(n_ranks):
+        for c, row in held[i].items():
+            out[corners[i]][corners[c]] = row
+    return [o.reshape(-1) for o in out]
+
+
 def sendrecv(xs: list, src: int, dst: int) -> list:
     out = [_bytes(x).copy() for x in xs]
     out[dst] = _bytes(xs[src]).copy()

@@ -133,7 +133,13 @@ def test_plan_geometry_without_a_gpu():
 
 @pytest.mark.parametrize("kw,err", [
     (dict(world=0), _lib.ERR_ARG), (dict(world=9), _lib.ERR_ARG),
-    (dict(op=10), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=12), _lib.ERR_ARG), (dict(protocol=2), _lib.ERR_ARG),
+    (dict(op=_lib.OP_HYPERCUBE_REDUCESCATTER, protocol=_lib.PROTO_SIMPLE, slot_bytes=448 << 10,
+          waves_per_channel_group=64), _lib.ERR_ARG),    # the hypercube kernels speak LL128 only
+    (dict(op=_lib.OP_HYPERCUBE_ALLGATHER, dtype=_lib.BYTES, world=6, slot_bytes=320 << 10,
+          waves_per_channel_group=64), _lib.ERR_ARG),    # 2^d corners
+    (dict(op=_lib.OP_HYPERCUBE_REDUCESCATTER, dtype=_lib.BYTES, slot_bytes=448 << 10,
+          waves_per_channel_group=64), _lib.ERR_ARG),    # a reduction needs a real dtype
     (dict(op=_lib.OP_ALLGATHER_TEMPORAL, dtype=_lib.BYTES, protocol=_lib.PROTO_SIMPLE,
           waves_per_channel_group=128), _lib.ERR_ARG),   # LL128 only
     (dict(op=_lib.OP_TREE_REDUCE, protocol=_lib.PROTO_SIMPLE, waves_per_channel_group=128),

@@ -189,8 +189,9 @@ def test_reference_style_self_tests_pass(monkeypatch, capsys, world, count):
     assert "equal: False" not in out
     # 3 point-to-point tests, broadcast, allgather, allreduce and alltoall on every
     # rank, reduce at the root, reducescatter on every rank; then the tree's
-    # broadcast on every rank and its reduce at the root
-    assert out.count("equal: True") == 3 + 4 * world + 1 + world + world + 1
+    # broadcast on every rank and its reduce at the root, the hypercube's
+    # reducescatter and allgather on every rank
+    assert out.count("equal: True") == 3 + 4 * world + 1 + world + world + 1 + 2 * world
 
 
 @pytest.mark.gpu

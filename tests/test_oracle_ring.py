@@ -167,6 +167,98 @@ def test_tree_reduce_properties(dt):
         assert np.array_equal(ring.to_float64(t, dt), np.sum(vals, axis=0, dtype=np.float64))
 
 
+def test_hand_computed_hypercube_order():
+    """Recursive halving: corner i adds the partner across the highest bit
+    first.  f16 near 2048 has a spacing of 2 and ties go to the even
+    significand: 2048 + 1 -> 2048, 2048 + 1.5 -> 2050, 2050 + 1 -> 2052,
+    2052 + 3 -> 2056."""
+    as_f = lambda raw, r, n: float(raw.view(np.float16).reshape(n, -1)[r, 0])
+
+    def buffers(n, row, values):
+        """Rank r's (n, 1) buffer: ``values[r]`` in row ``row``, zero elsewhere."""
+        out = []
+        for r in range(n):
+            b = np.zeros((n, 1), dtype=np.float16)
+            b[row, 0] = values[r]
+            out.append(b.view(np.uint8).reshape(-1))
+        return out
+
+    # four corners, row 0: (x0 + x2) + (x1 + x3) = (2048 + 1.5) + (1 + 0) = 2050 + 1 -> 2052;
+    # the ring ((2048 + 1) + 1.5) + 0, the binary tree (2048 + (1 + 0)) + 1.5 and halving
+    # from the lowest bit (2048 + 1) + (1.5 + 0) all give 2050
+    xs = buffers(4, 0, [2048.0, 1.0, 1.5, 0.0])
+    assert as_f(ring.hypercube_reducescatter(xs, "f16")[0], 0, 4) == 2052.0
+    assert as_f(ring.reducescatter(xs, "f16")[0], 0, 4) == 2050.0
+    assert float(ring.tree_fold([x[:2] for x in xs], [0, 1, 2, 3], "f16").view(np.float16)[0]) == 2050.0
+    # row 3: (x3 + x1) + (x2 + x0) = (2048 + 1.5) + (0 + 1) -> 2052
+    xs = buffers(4, 3, [1.0, 1.5, 0.0, 2048.0])
+    assert as_f(ring.hypercube_reducescatter(xs, "f16")[3], 3, 4) == 2052.0
+    # eight corners, row 0: ((x0 + x4) + (x2 + x6)) + ((x1 + x5) + (x3 + x7))
+    # = ((2048 + 1.5) + (1 + 0)) + ((1 + 1) + (1 + 0)) = (2050 + 1 -> 2052) + 3 -> 2056;
+    # the ring loses the ones: 2048 +1 +1 +1 -> 2048, + 1.5 -> 2050, + 1 -> 2052
+    xs = buffers(8, 0, [2048.0, 1.0, 1.0, 1.0, 1.5, 1.0, 0.0, 0.0])
+    assert as_f(ring.hypercube_reducescatter(xs, "f16")[0], 0, 8) == 2056.0
+    assert as_f(ring.reducescatter(xs, "f16")[0], 0, 8) == 2052.0
+    # row 5 = 0b101: ((x5 + x1) + (x7 + x3)) + ((x4 + x0) + (x6 + x2)), the same values
+    # moved to the corners that play these parts
+    vals = [0.0] * 8
+    for part, v in zip((5, 1, 7, 3, 4, 0, 6, 2), (2048.0, 1.5, 1.0, 0.0, 1.0, 1.0, 1.0, 0.0)):
+        vals[part] = v
+    assert as_f(ring.hypercube_reducescatter(buffers(8, 5, vals), "f16")[5], 5, 8) == 2056.0
+    # corners follow the ring: with ring 0 2 1 3 corner 1 is rank 2, so rank 2's row is
+    # (x[rank 2] + x[rank 3]) + (x[rank 0] + x[rank 1])  (corners 1, 3, 0, 2)
+    xs = buffers(4, 2, [1.0, 0.0, 2048.0, 1.5])
+    out = ring.hypercube_reducescatter(xs, "f16", [0, 2, 1, 3, 0])
+    assert as_f(out[2], 2, 4) == 2052.0
+    # only row r of rank r changes
+    assert all((out[r] == xs[r]).all() for r in (0, 1, 3))
+    # the operator's own account of the order (nested pairs of corner numbers)
+    from mintccl_amd import hypercube
+    assert hypercube.order(4, 0) == ((0, 2), (1, 3))
+    assert hypercube.order(8, 0) == (((0, 4), (2, 6)), ((1, 5), (3, 7)))
+    assert hypercube.order(8, 5) == (((5, 1), (7, 3)), ((4, 0), (6, 2)))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+def test_hypercube_properties(dt):
+    bits = 32 if dt == "f32" else 16
+    # two ranks: one commutative addition, the same as the ring's
+    x = [random_bits(2 * 3000, bits, 41 + r).view(np.uint8) for r in range(2)]
+    for mine, ringed in zip(ring.hypercube_reducescatter(x, dt), ring.reducescatter(x, dt)):
+        assert ring.same_values(mine, ringed, dt)
+    # small integers add exactly in any order
+    rng = np.random.default_rng(6)
+    for n in (4, 8):
+        vals = [rng.integers(-8, 9, (n, 500)).astype(np.float32) for _ in range(n)]
+        if dt == "f32":
+            raw = [v.view(np.uint8).reshape(-1) for v in vals]
+        elif dt == "f16":
+            raw = [v.astype(np.float16).view(np.uint8).reshape(-1) for v in vals]
+        else:
+            raw = [(v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(-1) for v in vals]
+        for perm in (None, [3, 1, 0, 2] + list(range(4, n)) + [3]):
+            mine = ring.hypercube_reducescatter(raw, dt, perm)
+            ringed = ring.reducescatter(raw, dt, perm)
+            for r in range(n):
+                assert ring.same_values(mine[r], ringed[r], dt)
+                got = ring.to_float64(mine[r], dt).reshape(n, -1)[r]
+                assert np.array_equal(got, np.sum([v[r] for v in vals], axis=0, dtype=np.float64))
+    with pytest.raises(ValueError):
+        ring.hypercube_reducescatter([x[0]] * 3, dt)
+
+
+def test_hypercube_allgather_is_allgather():
+    rng = np.random.default_rng(7)
+    for n in (1, 2, 4, 8):
+        xs = [rng.integers(0, 256, n * 96, dtype=np.uint8) for _ in range(n)]
+        for perm in (None, list(reversed(range(n))) + [n - 1]):
+            mine = ring.hypercube_allgather(xs, perm)
+            for a, b in zip(mine, ring.allgather(xs)):
+                assert np.array_equal(a, b)
+    with pytest.raises(ValueError):
+        ring.hypercube_allgather([xs[0]] * 6)
+
+
 def test_fold_order_with_a_permuted_ring():
     ring_ = [0, 2, 1, 3, 0]
     assert ring.fold_order(ring_, 1) == [1, 3, 0, 2]

@@ -58,11 +58,13 @@ def seats_for(d, deal):
 
 def all_seats(d):
     pipes = {_lib.OP_ALLGATHER: d.world, _lib.OP_REDUCESCATTER: d.world, _lib.OP_ALLREDUCE: d.world,
-             _lib.OP_ALLTOALL: d.world * d.world}.get(d.op, 1)
+             _lib.OP_ALLTOALL: d.world * d.world, _lib.OP_HYPERCUBE_REDUCESCATTER: d.world,
+             _lib.OP_HYPERCUBE_ALLGATHER: d.world}.get(d.op, 1)
     npos = {_lib.OP_SENDRECV: d.route_len, _lib.OP_BROADCAST: d.world, _lib.OP_ALLGATHER: d.world,
             _lib.OP_ALLGATHER_TEMPORAL: d.world, _lib.OP_TREE_BROADCAST: d.world,
             _lib.OP_TREE_REDUCE: d.world, _lib.OP_ALLREDUCE: 2 * d.world - 1,
-            _lib.OP_ALLTOALL: 2}.get(d.op, d.world + 1)
+            _lib.OP_ALLTOALL: 2, _lib.OP_HYPERCUBE_REDUCESCATTER: d.world,
+            _lib.OP_HYPERCUBE_ALLGATHER: d.world}.get(d.op, d.world + 1)
     threads = min(d.threads_per_block, d.waves_per_channel_group * 64)
     groups = -(-d.waves_per_channel_group * 64 // threads)
     return {(p, h, b) for p in range(pipes) for h in range(npos) for b in range(groups)}
@@ -106,6 +108,9 @@ CASES = [
          waves_per_channel_group=40, threads_per_block=64, root=1, **LOCAL),
     dict(op=_lib.OP_ALLREDUCE, count_bytes=16 << 20, slot_bytes=16 * 24 << 10, nslots=3,
          waves_per_channel_group=24, threads_per_block=192, **LOCAL),
+    # a hypercube: 8 rows x 8 corners
+    dict(op=_lib.OP_HYPERCUBE_REDUCESCATTER, count_bytes=8 << 20, slot_bytes=7 * 72 << 10, nslots=3,
+         waves_per_channel_group=72, threads_per_block=256, **LOCAL),
 ]
 
 
