@@ -123,19 +123,20 @@ typedef enum {
  * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
  * that gave up; word 2: step it waited for; word 3: abort flag polled by all
  * other waits.  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
- * then holds that number.  Error code 3: MINT_PLACE_LOCAL, and the device did
- * not deal the thread blocks evenly over its XCDs and compute units, so some
- * (channel, position) found no block: nothing has been stored into any input
- * or output buffer (a position waits for all seats to be taken before its
- * first such store), and the same launch with MINT_PLACE_SPREAD (cache_policy
- * 0) will do; after code 2 or 3 the staging is zeroed before it is used again
- * (the launch left seat counters behind).
+ * then holds that number.  Error code 3: MINT_PLACE_LOCAL, and a thread block
+ * found every seat of its XCD taken or waited in vain for its compute unit's
+ * number: the device did not deal an eighth of the grid to every XCD (blocks
+ * may be dealt over the compute units of an XCD in any way - a stream with a
+ * CU mask, compute units busy with other kernels, a grid that is resident in
+ * parts).  The same launch with MINT_PLACE_SPREAD (cache_policy 0) will do.
  * The words stay set until the caller zeroes them: every launch that finds
  * word 3 set gives up at its first wait (after at most 64 polls) and leaves
  * unspecified output, and only the first failure is recorded.  After a
- * non-zero word 0 the caller synchronises the stream, zeroes the block (the
- * staging needs no clearing: the next launch brings its own epoch) and treats
- * the outputs of every launch since the last clean check as lost.
+ * non-zero word 0 the caller synchronises the stream, zeroes the block and
+ * treats the outputs of every launch since the last clean check as lost;
+ * under MINT_PLACE_LOCAL it also zeroes the staging before it is used again
+ * (a launch that ends early can leave seat counters behind; the slots
+ * themselves need no clearing: the next launch brings its own epoch).
  * The reference has no abort path (common.py:106 is unused). */
 #define MINT_STATUS_WORDS 4
 
@@ -349,17 +350,22 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
  * by the code the kernels run.  The reference maps program_id to its work
  * directly (7_reducescatter.py:23-25: every rank is a GPU of its own); here a
  * block claims an entry of the list of the XCD it finds itself on: the
- * compute unit that was the `cu_rank`-th of XCD `xcd` to show up takes, with
- * its `nth` block (0-based), entry nth * 32 + cu_rank; blocks beyond a compute
- * unit's share and compute units beyond the 32nd draw a leftover ticket
- * (`leftover` = the ticket such a block would be handed; *used_leftover says
- * whether it was).  A launch of at most 32 entries per XCD (no compute unit
- * gets a second block) takes the whole list by that ticket.  Returns 1 and the seat (pipeline, position, block of the
- * position's group of thread blocks), 0 if the block has nothing to do, or a
- * negative mint_error.  Needs no GPU: the test of "every seat exactly once
- * for any arrival order". */
-int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, int leftover,
-                   int* used_leftover, int* pipeline, int* position, int* block_of_group);
+ * compute unit that was the `cu_rank`-th of XCD `xcd` to show up wants, with
+ * its `nth` block (0-based), entry nth * 32 + cu_rank; a block beyond a
+ * compute unit's share, of a compute unit beyond the 32nd, or whose entry is
+ * taken, draws a ticket and takes the first free entry from its ticket's
+ * place in the last, partial round (later tickets: from the head of the list)
+ * upwards.  A launch of at most 32 entries per XCD (no compute
+ * unit gets a second block) takes the whole list by ticket.  `state` is the
+ * XCD's counters, MINT_SEAT_STATE_WORDS words that the caller zeroes before
+ * the first block of a simulated launch and passes to every call for that
+ * XCD, in the order in which the blocks arrive.  Returns 1 and the seat
+ * (pipeline, position, block of the position's group of thread blocks), 0 if
+ * the block has nothing to do, or a negative mint_error.  Needs no GPU: the
+ * test of "every seat exactly once however the blocks are dealt". */
+#define MINT_SEAT_STATE_WORDS 17
+int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, uint64_t* state,
+                   int* pipeline, int* position, int* block_of_group);
 
 /* Validate and enqueue one fused launch that runs every rank's kernel: the
  * Triton launches kernel[(NUM_BLOCKS,)](recvbuff, sendbuff, inputbuff,

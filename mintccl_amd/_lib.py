@@ -27,7 +27,8 @@ MAX_EPOCH = 4095          # sector tags carry a 12-bit launch epoch
 (OK, ERR_ARG, ERR_ALIGN, ERR_GEOMETRY, ERR_RESIDENCY, ERR_HIP, ERR_TOO_LARGE,
  ERR_STAGING, ERR_NOT_READY) = 0, -1, -2, -3, -4, -5, -6, -7, -8
 VERSION = 102             # the interface version this binding was written for
-TICKET_BYTES = 18 * 1024  # the end of every rank's staging: room for the seat tickets
+TICKET_BYTES = 20 * 1024  # the end of every rank's staging: room for the seat tickets
+SEAT_STATE_WORDS = 17     # mint_ring_seat: counters of one XCD in a simulated launch
 BUILD_RING_STATS, BUILD_ROW_NOLOAD = 1, 2
 LAYOUT_PAIR, LAYOUT_WAVE64 = 0, 1
 F16, BF16, F32, BYTES = 0, 1, 2, 3
@@ -104,7 +105,7 @@ SYMBOLS = {
     "mint_ring_staging_bytes": (_sz, [_opp]),
     "mint_ring_grid_blocks": (_i, [_opp]),
     "mint_ring_schedule": (_i, [_opp, _i, _i, _i, _u32, _u32p, _u32p, _u32p, _u32p, _u32p]),
-    "mint_ring_seat": (_i, [_opp, _i, _i, _i, _i, _ip, _ip, _ip, _ip]),
+    "mint_ring_seat": (_i, [_opp, _i, _i, _i, ctypes.POINTER(ctypes.c_uint64), _ip, _ip, _ip]),
     "mint_ring_launch": (_i, [_opp, _vp]),
     "mint_ring_launch_debug": (_i, [_opp, _dbgp, _vp]),
     "mint_ring_launch_static": (_i, [_opp, _vp]),

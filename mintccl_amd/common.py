@@ -141,9 +141,8 @@ class RingTimeout(RuntimeError):
 
 class PlacementError(RuntimeError):
     """The local placement ran on a device that numbers its XCDs beyond 7
-    (status word 0 == 2) or that did not deal the thread blocks evenly over
-    its XCDs and compute units (status word 0 == 3; no caller buffer has been
-    written then)."""
+    (status word 0 == 2) or that did not deal an eighth of the thread blocks
+    to every XCD (status word 0 == 3)."""
 
 
 def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
@@ -572,23 +571,21 @@ class VirtualComm:
         if st[0] != 0:
             self.status.zero_()
             who = st[1]
-            if st[0] in (2, 3):
-                # a launch that could not seat all its blocks leaves its seat
-                # counters behind: start from cleared staging
-                self.staging.zero_()
-                self.epoch = 0
-                if self.epoch_word is not None:
-                    self.epoch_word.zero_()
+            # a launch that ends early can leave its seat counters behind:
+            # start from cleared staging
+            self.staging.zero_()
+            self.epoch = 0
+            if self.epoch_word is not None:
+                self.epoch_word.zero_()
             if st[0] == 2:
                 raise PlacementError(
                     f"a block ran on XCD {st[2]}: the local placement deals work to XCDs 0..7; "
                     "use placement spread (and cache_policy 0) on this device")
             if st[0] == 3:
                 raise PlacementError(
-                    "the device did not deal the thread blocks evenly over its XCDs and compute "
-                    "units, so a (channel, position) of the local placement found no block; no "
-                    "input or output buffer has been written - run the launch again with "
-                    "placement spread (and cache_policy 0)")
+                    "the device did not deal an eighth of the thread blocks to every XCD, so a "
+                    "block of the local placement found no seat; outputs are unspecified - use "
+                    "placement spread (and cache_policy 0) on this stream")
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
                 f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]} "

@@ -207,16 +207,11 @@ __device__ __forceinline__ void hyper_walk(const RingArgs& a, const int p, const
 // placement a wave-channel's whole tree shares one XCD.
 template <int DT, int CPI>
 __global__ void __launch_bounds__(512) hyper_kernel(const RingArgs a) {
-    __shared__ int entry[2];
+    __shared__ int entry[1];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
-    // a node that writes a caller's buffer (the owner of a reduced row, everybody
-    // else in an allgather) first makes sure every node has a thread block
-    const bool saves = a.op == OP_HYPER_REDUCESCATTER ? st.h == (int)a.start[st.p]
-                                                      : st.h != (int)a.start[st.p];
-    if (saves && !seats_confirmed(a, st.sequence)) return;
     hyper_walk<DT, CPI>(a, st.p, st.h, st.w);
 }
 

@@ -307,6 +307,10 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
             plan->blocks = kXcds * kCusPerXcd * (r0 > r1 ? r0 : r1);
         }
     }
+    // (the map through which blocks claim their seats holds 1024 entries per XCD:
+    // more thread blocks than a device keeps resident)
+    if (op->placement == MINT_PLACE_LOCAL && plan->blocks / kXcds > kSeatWords * 64)
+        return MINT_ERR_RESIDENCY;
     plan->unroll = a.k_per_wave % 4 == 0 ? 4 : (a.k_per_wave % 2 == 0 ? 2 : 1);
     // Every rank's staging ends in room for the counters the blocks of a launch
     // under the local placement claim their seats through (those of the first
@@ -711,25 +715,32 @@ int mint_ring_schedule(const mint_ring_op* op, int pipeline, int position, int w
     }
 }
 
-int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, int leftover,
-                   int* used_leftover, int* pipeline, int* position, int* block_of_group) {
+int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, uint64_t* state,
+                   int* pipeline, int* position, int* block_of_group) {
     Plan plan;
     const int err = make_plan(op, &plan);
     if (err != MINT_OK) return err;
     if (plan.empty || op->placement != MINT_PLACE_LOCAL || xcd < 0 || xcd >= kXcds || cu_rank < 0 ||
-        nth < 0 || leftover < 0)
+        nth < 0 || !state)
         return MINT_ERR_ARG;
     const SeatList list = seat_list(plan.args, plan.blocks);
-    bool used = false;
+    uint64_t* const taken = state;
+    uint64_t& tickets = state[kSeatWords];
     int y;
     if (seats_in_order_of_arrival(plan.args, list)) {
-        // taken in the order of arrival at one counter per XCD: `leftover` is that ticket
-        used = true;
-        y = leftover < list.len ? leftover : -1;
+        // taken in the order of arrival at one counter per XCD
+        y = tickets < (uint64_t)list.len ? (int)tickets : -1;
+        ++tickets;
     } else {
-        y = seat_entry(list, cu_rank, nth, leftover, used);
+        y = seat_claim(
+            list, seat_wanted(list, cu_rank, nth),
+            [&](int word, uint64_t bits) {
+                const uint64_t before = taken[word];
+                taken[word] |= bits;
+                return before;
+            },
+            [&]() { return (int)tickets++; });
     }
-    if (used_leftover) *used_leftover = used ? 1 : 0;
     int p = 0, h = 0, gw = 0;
     if (y < 0 || !seat_of_entry(plan.args, xcd, y, p, h, gw)) return 0;
     if (pipeline) *pipeline = p;

@@ -167,7 +167,6 @@ __device__ __forceinline__ bool wait_count(const uint64_t* word, uint32_t epoch,
 constexpr int kCusPerXcd = 32;      // MI355X: 256 CUs in 8 XCDs
 struct Seat {
     int p, h, gw, w;
-    uint32_t sequence;      // local placement: sequence number of the launch (seats_confirmed)
     bool ok;
 };
 __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int wib) {
@@ -188,14 +187,15 @@ __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int
 // (channel, position).  Which entry a thread block takes does not depend on
 // its number: the block asks the hardware where it runs (XCC_ID, and the
 // compute unit's number from HW_ID) and claims an entry through counters in
-// device memory.  Any order in which the device deals its blocks over XCDs
-// and compute units gives every entry to exactly one block, provided every
-// XCD receives an eighth of the grid and every compute unit its share of
-// that; if not, entries stay unclaimed, no position stores into a caller's
-// buffer (seats_confirmed below) and the launch reports status 3.
+// device memory.  Every block gets an entry, and every entry goes to exactly
+// one block, whatever way the device deals its blocks over the compute units
+// of an XCD (a stream confined to some of them, compute units busy with
+// another stream's kernel, a grid that is only partly resident at any time),
+// provided every XCD receives an eighth of the grid; a block that finds its
+// XCD's list taken ends the launch with status 3.
 //
 // The list of an XCD is walked in rounds of one entry per compute unit: the
-// compute unit that was the j-th of its XCD to show up takes, with its n-th
+// compute unit that was the j-th of its XCD to show up wants, with its n-th
 // block, entry n * 32 + j.  All blocks of a compute unit so share j, and the
 // order of the list decides what a compute unit holds: with h = y % npos and
 // a position count that divides 32 (8 ranks) every compute unit holds blocks
@@ -205,38 +205,47 @@ __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int
 // walks are fastest that way (an allgather whose compute units hold a mix of
 // positions takes 4 - 10 % longer; the order in which blocks reach a counter
 // is nothing like the order of their numbers, so one counter per XCD would
-// mix them).  Entries of a last, partial round (a list that is no multiple of
-// 32) and blocks beyond a compute unit's share go through one more counter
-// per XCD, the leftover tickets.
+// mix them).  An entry is claimed by setting its bit in the XCD's map of
+// taken entries; a block that wants none (a last, partial round of a list
+// that is no multiple of 32; a compute unit that got more than its share; a
+// 33rd compute unit) or finds its entry taken draws a ticket: the first
+// `rest` tickets start at their entry of the partial round, all later ones at
+// the head of the list, and a block takes the first free entry from there
+// upwards.  With every compute unit at its share that is one look at the
+// partial round each; with any other deal the blocks sort themselves out - as
+// many blocks as entries, so there is a free one for everybody - and only the
+// neat division of positions over compute units is lost.  (From the head
+// upwards, because a list is also the order in which channels become
+// complete: where not all blocks are resident at once - half of the compute
+// units masked off - the blocks that are there have to fill whole channels,
+// lowest first, or they wait for blocks that cannot start.)
 //
 // The counters (64-bit words in device memory, zero between launches):
 //   xcd * 2048 + cu * 8     per compute unit: blocks that have arrived in bits
 //                           23:0, j + 1 in bits 31:24 once it is known
 //   16384 + xcd * 128       per XCD, a line of its own: + 0 compute units
-//                           registered, + 8 leftover tickets handed out, + 16
-//                           entries claimed
-//   17408, 17416            XCDs whose list is claimed completely, for launches
-//                           of even / odd sequence number
-//   17536                   sequence number of the launch (a line of its own)
+//                           registered, + 8 tickets handed out, + 16 entries
+//                           claimed
+//   18432 + xcd * 128       per XCD, a line of its own: the map of taken
+//                           entries, 1024 bits
 // A line that blocks of several XCDs work on is slow (a counter per XCD in one
 // line: 40 - 60 us for 160 blocks per XCD; in lines of their own: 6 us), hence
 // the spacing.  The block that claims the last entry of its XCD's list puts
 // that XCD's counters back to zero, so a launch finds them as the launch
-// before left them - zero - and the common path is one atomic add per counter
+// before left them - zero - and the common path is one atomic per counter
 // (with the launch epoch in every word instead, every block of a launch found
 // a stale word first and went through a compare-and-swap: three more trips).
-// The count of complete XCDs is looked at long after it was counted up
-// (positions check it before their first store into a caller's buffer), so it
-// is not put back by its own launch: there are two, used in turn - the block
-// that counts the eighth XCD clears the other one and moves the sequence
-// number on, which every block reads when it starts.  A launch that could not
-// seat all its blocks (status 2 or 3) leaves counters behind: the staging is
-// cleared before it is used again.  All of these are atomics and loads at
-// agent scope: one place serves them whichever XCD asks.
-constexpr uint32_t kTicketXcdLine = 16384, kTicketXcdStride = 128, kTicketComplete = 17408,
-                   kTicketSequence = 17536;
-constexpr uint32_t kTicketBytes = 18 * 1024;
+// Nothing waits for the whole grid to be seated: a launch whose blocks are
+// not all resident at once (a stream confined to half of the compute units)
+// runs the channels that are complete, and their blocks make room for the
+// rest.  A launch that could not seat all its blocks (status 2 or 3) leaves
+// counters behind: the staging is cleared before it is used again.  All of
+// these are atomics and loads at agent scope: one place serves them whichever
+// XCD asks.
+constexpr uint32_t kTicketXcdLine = 16384, kTicketXcdStride = 128, kTicketTaken = 18432;
+constexpr uint32_t kTicketBytes = 20 * 1024;
 constexpr uint32_t kSeatPatience = 1u << 18;
+constexpr int kSeatWords = 16;            // map of taken entries: 1024 per XCD at most
 
 // The list of one XCD: `len` entries, of which the first `full` rounds are
 // taken by (compute unit, arrival) and the `rest` after them by leftover ticket.
@@ -250,15 +259,39 @@ __host__ __device__ __forceinline__ SeatList seat_list(const RingArgs& a, int gr
     l.rest = l.len % kCusPerXcd;
     return l;
 }
-// Entry for the block that arrived `nth` on the compute unit registered as
-// `j`-th of its XCD; `leftover` = the ticket it would get from the XCD's
-// leftover counter, `used` says whether it took it.  -1: nothing to claim.
-__host__ __device__ __forceinline__ int seat_entry(const SeatList& l, int j, int nth, int leftover,
-                                                   bool& used) {
-    used = false;
-    if (j < kCusPerXcd && nth < l.full) return nth * kCusPerXcd + j;
-    used = true;
-    return leftover < l.rest ? l.full * kCusPerXcd + leftover : -1;
+// Entry the block that arrived `nth` on the compute unit registered as `j`-th
+// of its XCD wants; -1: none, it draws a ticket.
+__host__ __device__ __forceinline__ int seat_wanted(const SeatList& l, int j, int nth) {
+    return j < kCusPerXcd && nth < l.full ? nth * kCusPerXcd + j : -1;
+}
+// Claims `wanted`, or - with -1 or the entry taken - a free entry by ticket:
+// ticket t < rest starts at entry t of the partial round, every later one at
+// entry 0, and takes the first free entry from there upwards (round the list).
+// `fetch_or(word, bits)` sets bits in word `word` of the XCD's map of taken
+// entries and returns what the word held before; `draw()` hands out the next
+// ticket.  -1: no entry is free (more blocks than entries).
+template <class FetchOr, class Draw>
+__host__ __device__ __forceinline__ int seat_claim(const SeatList& l, int wanted, FetchOr fetch_or,
+                                                   Draw draw) {
+    if (wanted >= 0 && !((fetch_or(wanted >> 6, 1ull << (wanted & 63)) >> (wanted & 63)) & 1ull))
+        return wanted;
+    const int t = draw();
+    int e = t < l.rest ? l.full * kCusPerXcd + t : 0;
+    const int last_word = (l.len - 1) >> 6;
+    // (every miss means that another block took an entry, so len looks and a
+    // walk over the words suffice)
+    for (int looks = 0; looks < l.len + 2 * kSeatWords; ++looks) {
+        const int word = e >> 6, bit = e & 63;
+        const uint64_t before = fetch_or(word, 1ull << bit);
+        if (!((before >> bit) & 1ull)) return e;
+        // the lowest entry of this word above e that was free a moment ago
+        uint64_t free_above = ~before & ~((2ull << bit) - 1ull);
+        if (bit == 63) free_above = 0;
+        if (word == last_word && (l.len & 63)) free_above &= (1ull << (l.len & 63)) - 1ull;
+        if (free_above) e = word * 64 + __builtin_ctzll(free_above);
+        else e = word < last_word ? (word + 1) * 64 : 0;
+    }
+    return -1;
 }
 // A list of at most one round (a small launch: no compute unit gets a second
 // block) is simply taken in the order in which the blocks reach one counter:
@@ -328,11 +361,8 @@ __device__ __forceinline__ uint64_t ticket_add(uint64_t* word, uint64_t v) {
 // counters back to zero: reset_tickets).  The wait here is for another block to
 // be dispatched, not for data: it gets at least kSeatPatience looks whatever
 // budget the caller gave the data waits.
-__device__ __forceinline__ int claim_entry(const RingArgs& a, uint32_t& sequence, int& xcd,
-                                           bool& last) {
+__device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& last) {
     last = false;
-    // (in flight together with the first atomic below)
-    const uint64_t seq_word = ld64_agent(ticket_word(a, kTicketSequence));
     xcd = xcc_id();
     if (xcd >= kXcds) {
         report_error(a.status, 2, 0, 0, 0, (uint64_t)xcd);
@@ -371,83 +401,57 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, uint32_t& sequence
             }
             jfield &= 0xFFu;
         }
-        bool wants_leftover;
-        y = seat_entry(list, (int)jfield - 1, (int)nth, 0, wants_leftover);
-        if (wants_leftover)
-            y = seat_entry(list, (int)jfield - 1, (int)nth, (int)ticket_add(line + 1, 1ull),
-                           wants_leftover);
-        if (y < 0) return -1;
+        uint64_t* const taken = ticket_word(a, kTicketTaken + (uint32_t)xcd * kTicketXcdStride);
+        y = seat_claim(
+            list, seat_wanted(list, (int)jfield - 1, (int)nth),
+            [&](int word, uint64_t bits) {
+                return (uint64_t)__hip_atomic_fetch_or((MINT_GLOBAL unsigned long long*)(taken + word),
+                                                       (unsigned long long)bits, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+            },
+            [&]() { return (int)ticket_add(line + 1, 1ull); });
+        if (y < 0) {
+            report_error(a.status, 3, 0, 0, 0, (uint64_t)cu);
+            return -1;
+        }
         claimed = (uint32_t)ticket_add(line + 2, 1ull);
     }
-    sequence = (uint32_t)seq_word;
     if (y < 0) return -1;
-    // the block that claims the last entry of its XCD says so to everybody; the
-    // one that does so for the last XCD prepares the counter of the next launch
-    if (claimed + 1u == (uint32_t)list.len) {
-        last = true;
-        uint64_t* const complete = ticket_word(a, kTicketComplete);
-        if (ticket_add(complete + (sequence & 1u), 1ull) + 1u == (uint64_t)kXcds) {
-            __hip_atomic_store((MINT_GLOBAL unsigned long long*)(complete + ((sequence & 1u) ^ 1u)), 0ull,
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            (void)ticket_add(ticket_word(a, kTicketSequence), 1ull);
-        }
-    }
+    // the block that claims the last entry of its XCD's list clears up
+    last = claimed + 1u == (uint32_t)list.len;
     return y;
 }
 // Puts the counters of XCD `xcd` back to zero (the thread block that claimed
 // the last entry of the XCD's list; every other claim of the launch on this
 // XCD has been counted by then).
 __device__ __forceinline__ void reset_tickets(const RingArgs& a, int xcd) {
-    for (uint32_t i = threadIdx.x; i < 256u + 3u; i += blockDim.x) {
-        uint64_t* const w = i < 256u ? ticket_word(a, (uint32_t)xcd * 2048u + i * 8u)
-                                     : ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride) +
-                                           (i - 256u);
+    for (uint32_t i = threadIdx.x; i < 256u + 3u + (uint32_t)kSeatWords; i += blockDim.x) {
+        uint64_t* const w =
+            i < 256u ? ticket_word(a, (uint32_t)xcd * 2048u + i * 8u)
+            : i < 259u ? ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride) + (i - 256u)
+                       : ticket_word(a, kTicketTaken + (uint32_t)xcd * kTicketXcdStride) + (i - 259u);
         __hip_atomic_store((MINT_GLOBAL unsigned long long*)w, 0ull, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
 }
-// Before a position stores into a caller's buffer for the first time: every
-// entry of every XCD's list has been claimed, so every (channel, position) of
-// the launch is being served.  Bounded; false (status 3) otherwise - then no
-// caller buffer has been written and the caller can run the launch again
-// with the spread placement.
-__device__ __forceinline__ bool seats_confirmed(const RingArgs& a, uint32_t sequence) {
-    if (a.placement != PLACE_LOCAL) return true;
-    const uint64_t* const word = ticket_word(a, kTicketComplete) + (sequence & 1u);
-    const uint32_t budget = a.spin_budget < kSeatPatience ? kSeatPatience : a.spin_budget;
-    for (uint32_t spins = 0;; ++spins) {
-        const uint32_t n = __builtin_amdgcn_readfirstlane((uint32_t)ld64_agent(word));
-        if (n == (uint32_t)kXcds) return true;
-        if (spins >= budget || ((spins & 63u) == 63u && aborted(a.status))) {
-            report_error(a.status, 3, 0, 0, 0, (uint64_t)n);
-            return false;
-        }
-        __builtin_amdgcn_s_sleep(2);
-    }
-}
-
 // The seat of this wavefront.  Under the local placement wavefront 0 of the
 // thread block claims the block's entry and hands it to the others through
-// `shared_entry` (two ints of LDS): every wavefront of the block has to call.
+// `shared_entry` (an int of LDS): every wavefront of the block has to call.
 __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib, int wave_of_block,
                                           MINT_LDS int* shared_entry) {
     // (locals, not members of the result: a member passed by reference keeps
     // the whole struct in scratch memory)
     int p = 0, h = 0, gw = 0;
-    uint32_t sequence = 0;
     bool seated = true;
     if (a.placement == PLACE_LOCAL) {
         if (wave_of_block == 0 && lane_id() == 0) {       // one lane: the counters count blocks
             int xcd = 0;
             bool last = false;
-            uint32_t seq = 0;
-            const int y = claim_entry(a, seq, xcd, last);
+            const int y = claim_entry(a, xcd, last);
             shared_entry[0] = y < 0 ? -1 : (y * kXcds + xcd) * 2 + (last ? 1 : 0);
-            shared_entry[1] = (int)(seq & 1u);
         }
         __syncthreads();
         const int e = __builtin_amdgcn_readfirstlane(shared_entry[0]);
-        sequence = (uint32_t)__builtin_amdgcn_readfirstlane(shared_entry[1]);
         if (e >= 0 && (e & 1)) reset_tickets(a, (e >> 1) % kXcds);
         seated = e >= 0 && seat_of_entry(a, (e >> 1) % kXcds, (e >> 1) / kXcds, p, h, gw);
     } else {
@@ -459,7 +463,6 @@ __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib, i
     }
     Seat st;
     st.p = p; st.h = h; st.gw = gw; st.w = 0;
-    st.sequence = sequence;
     st.ok = false;
     if (!seated || gw * wpb + wib >= a.waves) return st;
     st.w = seat_wave(a, gw, wpb, wib);
@@ -1275,7 +1278,7 @@ template <int PROTO, int DT, int CPI, int U>
 __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     // the wave index is the same in every lane: keep it (and all the index
     // arithmetic that hangs off it) in scalar registers
-    __shared__ int entry[2];
+    __shared__ int entry[1];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
@@ -1286,7 +1289,6 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     const Role role = role_of(a, p, h);
     // a position that writes a caller's buffer first makes sure that every
     // (channel, position) of the launch has a thread block
-    if (role.save && !seats_confirmed(a, st.sequence)) return;
     walk_as<PROTO, DT, CPI, U, false>(a, p, h, w, role);
 }
 
@@ -1403,7 +1405,7 @@ template <int DT, int CPI, int U, int WPB, int R>
 __global__ void __launch_bounds__((WPB + 1) * 64) ring_kernel_lds(const RingArgs a) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     MINT_LDS uint8_t* lds = (MINT_LDS uint8_t*)lds_raw;
-    __shared__ int entry[2];
+    __shared__ int entry[1];
     if (threadIdx.x < 16) reinterpret_cast<MINT_LDS uint32_t*>(lds)[threadIdx.x] = 0u;
     __syncthreads();
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
@@ -1415,7 +1417,6 @@ __global__ void __launch_bounds__((WPB + 1) * 64) ring_kernel_lds(const RingArgs
         if (role.load) row_fetcher<U, WPB, R>(a, st, role, lds);
         return;
     }
-    if (role.save && !seats_confirmed(a, st.sequence)) return;
     walk_as<PROTO_LL128, DT, CPI, U, true>(a, st.p, st.h, st.w, role,
                                            lds_port(lds, wib, a.fetch_depth, U));
 }

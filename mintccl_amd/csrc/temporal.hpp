@@ -284,14 +284,11 @@ __device__ __forceinline__ void temporal_walk(const RingArgs& a, const int h, co
 // Seats are dealt as for the ring kernels.
 template <int CPI>
 __global__ void __launch_bounds__(512) temporal_kernel(const RingArgs a) {
-    __shared__ int entry[2];
+    __shared__ int entry[1];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
-    // (every position but the origins' writes the buffers of the ranks it
-    // serves: first make sure every position of the launch has a thread block)
-    if (st.h != 0 && !seats_confirmed(a, st.sequence)) return;
     temporal_walk<CPI>(a, st.h, st.w);
 }
 

@@ -254,14 +254,11 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
 // with the local placement a wave-channel's whole tree shares one XCD.
 template <int DT, int CPI>
 __global__ void __launch_bounds__(512) tree_kernel(const RingArgs a) {
-    __shared__ int entry[2];
+    __shared__ int entry[1];
     const int wpb = (int)(blockDim.x >> 6);
     const int wib = (int)__builtin_amdgcn_readfirstlane((uint32_t)wave_in_block());
     const Seat st = take_seat(a, wpb, wib, wib, (MINT_LDS int*)entry);
     if (!st.ok) return;
-    // a node that writes a caller's buffer (the root of a reduce, everybody
-    // else in a broadcast) first makes sure every node has a thread block
-    if ((a.op == OP_TREE_REDUCE ? st.h == 0 : st.h != 0) && !seats_confirmed(a, st.sequence)) return;
     tree_walk<DT, CPI>(a, st.h, st.w);
 }
 

@@ -352,6 +352,52 @@ def test_captured_collectives_replay(dev):
 
 
 @pytest.mark.gpu
+def test_local_placement_on_a_stream_confined_to_half_of_the_compute_units(dev):
+    """Thread blocks claim their seats whatever compute units they land on: on
+    a stream with a CU mask every compute unit in use gets twice its share of
+    the blocks, and the launches (several rounds over the compute units, with
+    and without compute units set apart for origins) still seat every block."""
+    import ctypes
+    from mintccl_amd import _lib
+    from mintccl_amd.allgather import allgather
+    from mintccl_amd.common import VirtualComm
+    from mintccl_amd.reducescatter import reducescatter
+    hip = ctypes.CDLL("libamdhip64.so")
+    words = (ctypes.c_uint32 * 8)(*([0x00FF00FF] * 8))
+    handle = ctypes.c_void_p()
+    assert hip.hipExtStreamCreateWithCUMask(ctypes.byref(handle), 8, words) == 0
+    stream = torch.cuda.ExternalStream(handle.value)
+    world, n = 8, 100003
+    comm = VirtualComm(world_size=world, device=dev, spin_budget=4000000)
+    assert comm.placement == _lib.PLACE_LOCAL
+    host = rank_rows(world, n, "f16", 8100)
+    bufs = [h.to(dev) for h in host]
+    torch.cuda.synchronize(dev)
+    with torch.cuda.stream(stream):
+        for _ in range(2):          # the second launch finds the counters as the first left them
+            for b, h in zip(bufs, host):
+                b.copy_(h, non_blocking=False)
+            comm.run(lambda r: reducescatter(bufs[r], comm))
+            assert comm.last_grid >= 8 * 64
+        comm.check()
+        want = ring.reducescatter([as_bytes(h) for h in host], "f16")
+        assert all(np.array_equal(as_bytes(b), w) for b, w in zip(bufs, want))
+        comm.run(lambda r: allgather(bufs[r], comm))
+        assert comm.last_grid >= 8 * 64
+        comm.check()
+        for b, w in zip(bufs, ring.allgather(want)):
+            assert np.array_equal(as_bytes(b), w)
+    # and the same communicator on an ordinary stream afterwards
+    for b, h in zip(bufs, host):
+        b.copy_(h)
+    comm.run(lambda r: reducescatter(bufs[r], comm))
+    comm.check()
+    assert all(np.array_equal(as_bytes(b), w) for b, w in zip(bufs, want))
+    torch.cuda.synchronize(dev)
+    assert hip.hipStreamDestroy(handle) == 0
+
+
+@pytest.mark.gpu
 def test_captured_ll128_launch_replayed_after_an_eager_simple_launch(dev):
     """A communicator with its epoch in device memory: an LL128 allgather is
     captured while the launch before it was LL128 too; between the replays an

@@ -3,16 +3,17 @@ position, thread block of the position's group) a block takes, listed on the
 host by the code the kernels run (``mint_ring_seat``).  No GPU needed.
 
 A block claims an entry of the list of the XCD it finds itself on through
-counters: the compute unit that was the j-th of its XCD to show up takes, with
-its n-th block, entry n * 32 + j; what is left goes by leftover ticket.  The
-reference has nothing of the kind (``7_reducescatter.py:23-25`` maps
-``program_id`` to its work directly: every rank is a GPU of its own).  What
-has to hold: whatever order the device deals its blocks in - over the XCDs,
-over the compute units of an XCD, and whatever order they reach the counters
-in - every seat is taken exactly once, as long as every XCD receives an
-eighth of the grid and every compute unit its share of that; and when a
-compute unit falls short, a seat stays empty (which the kernels detect before
-anything is stored into a caller's buffer)."""
+counters: the compute unit that was the j-th of its XCD to show up wants, with
+its n-th block, entry n * 32 + j; a block that wants none, or finds its entry
+taken, draws a ticket and takes the first free entry from the ticket's place
+in the last, partial round (later tickets: from the head of the list) upwards.  The reference has nothing of the kind
+(``7_reducescatter.py:23-25`` maps ``program_id`` to its work directly: every
+rank is a GPU of its own).  What has to hold: whatever way the device deals
+its blocks - over the compute units of an XCD (all 32, half of them on a
+stream with a CU mask, some of them busy with another kernel), and whatever
+order they reach the counters in - every seat is taken exactly once, as long
+as every XCD receives an eighth of the grid; and with every compute unit at
+its share, a compute unit holds the entries of its own column."""
 import ctypes
 import random
 
@@ -32,7 +33,7 @@ def op_for(**kw):
     return d
 
 
-def seats_for(d, deal):
+def seats_for(d, deal, with_cu=False):
     """Simulate a launch: `deal(xcd, count)` returns, for the `count` blocks an
     XCD receives, the hardware compute unit of each in the order in which they
     reach the counters.  Returns the list of seats taken."""
@@ -41,19 +42,41 @@ def seats_for(d, deal):
     assert grid > 0 and grid % XCDS == 0
     taken = []
     for xcd in range(XCDS):
-        rank_of, arrived, leftover = {}, {}, 0
+        rank_of, arrived = {}, {}
+        state = (ctypes.c_uint64 * _lib.SEAT_STATE_WORDS)()
         for cu in deal(xcd, grid // XCDS):
             j = rank_of.setdefault(cu, len(rank_of))
             n = arrived.get(cu, 0)
             arrived[cu] = n + 1
-            used, p, h, b = (ctypes.c_int(0) for _ in range(4))
-            rc = L.mint_ring_seat(d, xcd, j, n, leftover, ctypes.byref(used), ctypes.byref(p),
-                                  ctypes.byref(h), ctypes.byref(b))
+            p, h, b = (ctypes.c_int(0) for _ in range(3))
+            rc = L.mint_ring_seat(d, xcd, j, n, state, ctypes.byref(p), ctypes.byref(h),
+                                  ctypes.byref(b))
             assert rc in (0, 1), rc
-            leftover += used.value
             if rc == 1:
-                taken.append((p.value, h.value, b.value))
+                taken.append((p.value, h.value, b.value) if not with_cu else
+                             (p.value, h.value, b.value, cu))
     return taken
+
+
+def L_grid(d):
+    return _lib.lib().mint_ring_grid_blocks(d)
+
+
+def seats_for_xcd(d, xcd, cus):
+    """One XCD of a simulated launch: (pipeline, position, block, compute unit) per seat."""
+    L = _lib.lib()
+    rank_of, arrived, out = {}, {}, []
+    state = (ctypes.c_uint64 * _lib.SEAT_STATE_WORDS)()
+    for cu in cus:
+        j = rank_of.setdefault(cu, len(rank_of))
+        n = arrived.get(cu, 0)
+        arrived[cu] = n + 1
+        p, h, b = (ctypes.c_int(0) for _ in range(3))
+        rc = L.mint_ring_seat(d, xcd, j, n, state, ctypes.byref(p), ctypes.byref(h), ctypes.byref(b))
+        assert rc in (0, 1), rc
+        if rc == 1:
+            out.append((p.value, h.value, b.value, cu))
+    return out
 
 
 def all_seats(d):
@@ -141,15 +164,106 @@ def uneven(xcd_short):
     return deal
 
 
-def test_a_compute_unit_that_falls_short_leaves_seats_empty():
-    # a tree reduce: 8 positions, 128 entries per XCD = 4 rounds over the compute
-    # units.  The compute unit that gets two blocks too few leaves two entries
-    # unclaimed (the kernels then report status 3 before any caller buffer is
-    # written); nothing is taken twice
-    d = op_for(**CASES[3])
-    taken = seats_for(d, uneven(3))
-    assert len(taken) == len(set(taken))
-    assert len(set(taken)) == len(all_seats(d)) - 2
+def masked(keep):
+    """A stream confined to `keep` of the 32 compute units of every XCD: they
+    take the XCD's blocks in turn, and reach the counters in any order."""
+    def deal(xcd, count):
+        cus = [(i % keep) * 3 + 1 for i in range(count)]
+        random.Random(100 + xcd).shuffle(cus)
+        return cus
+    return deal
+
+
+def crowded(xcd, count):
+    """Another kernel occupies most of eleven compute units: they take one
+    block each, the others share the rest, and one takes a third of the grid."""
+    cus = list(range(11)) + [11] * (count // 3)
+    cus += [12 + i % 20 for i in range(count - len(cus))]
+    random.Random(7 + xcd).shuffle(cus)
+    return cus
+
+
+@pytest.mark.parametrize("kw", CASES)
+def test_every_seat_exactly_once_however_uneven_the_deal(kw):
+    d = op_for(**kw)
+    want = all_seats(d)
+    for deal in (uneven(3), masked(16), masked(8), masked(24), masked(5), masked(1), crowded):
+        taken = seats_for(d, deal)
+        assert len(taken) == len(set(taken)), "a seat was taken twice"
+        assert set(taken) == want
+
+
+def test_with_every_compute_unit_at_its_share_a_compute_unit_holds_one_position():
+    # 8 positions, 32 compute units: the entries of a compute unit's column all
+    # have the same position, whatever order the blocks reach the counters in;
+    # with compute units set apart for the origins, those hold origins only and
+    # no other holds one (what the copying collectives' speed rests on)
+    for origin_cus in (0, 9):
+        d = op_for(**{**CASES[1], "origin_cus": origin_cus})
+        per_xcd = L_grid(d) // XCDS
+        assert per_xcd % CUS == 0           # whole rounds: nothing is dealt by ticket
+        for deal in (in_turn(list(range(CUS))), shuffled(1), shuffled(2)):
+            by_cu, taken = {}, []
+            for xcd in range(XCDS):
+                one = seats_for_xcd(d, xcd, deal(xcd, per_xcd))
+                for p, h, b, cu in one:
+                    by_cu.setdefault((xcd, cu), []).append(h)
+                taken += one
+            assert len(taken) == len({t[:3] for t in taken})
+            for hs in by_cu.values():
+                if origin_cus:
+                    assert all(h == 0 for h in hs) or all(h != 0 for h in hs), hs
+                else:
+                    assert len(set(hs)) == 1, hs
+            if origin_cus:
+                assert sum(all(h == 0 for h in hs) for hs in by_cu.values()) == XCDS * origin_cus
+
+
+@pytest.mark.parametrize("case,cus,per_cu", [(0, 16, 12), (0, 8, 16), (1, 16, 5), (3, 16, 6),
+                                             (8, 16, 5), (0, 32, 6), (0, 21, 9)])
+def test_a_partly_resident_grid_fills_whole_channels(case, cus, per_cu):
+    """Where not all blocks of a launch are resident at once (a stream confined
+    to `cus` compute units that hold `per_cu` thread blocks each), the blocks
+    that are there have to complete channels - every position of a (pipeline,
+    block of the group) - so that these finish and make room: played per XCD
+    with blocks dealt to the compute units in turn as room becomes free."""
+    d = op_for(**CASES[case])
+    L = _lib.lib()
+    per_xcd = L.mint_ring_grid_blocks(d) // XCDS
+    npos = max(h for _, h, _ in all_seats(d)) + 1
+    for xcd in range(XCDS):
+        state = (ctypes.c_uint64 * _lib.SEAT_STATE_WORDS)()
+        rank_of, arrived = {}, {}
+        room = {c * 2 + 1: per_cu for c in range(cus)}
+        members, holder = {}, {}
+        pending, turn, seated = per_xcd, 0, 0
+        while pending or members:
+            progressed = False
+            for _ in range(cus):                         # one round of dispatch
+                cu = list(room)[turn % cus]
+                turn += 1
+                if pending and room[cu]:
+                    j = rank_of.setdefault(cu, len(rank_of))
+                    n = arrived.get(cu, 0)
+                    arrived[cu] = n + 1
+                    p, h, b = (ctypes.c_int(0) for _ in range(3))
+                    rc = L.mint_ring_seat(d, xcd, j, n, state, ctypes.byref(p), ctypes.byref(h),
+                                          ctypes.byref(b))
+                    assert rc in (0, 1)
+                    pending -= 1
+                    progressed = True
+                    if rc == 1:                         # (an empty entry: the block exits at once)
+                        room[cu] -= 1
+                        seated += 1
+                        members.setdefault((p.value, b.value), set()).add(h.value)
+                        holder.setdefault((p.value, b.value), []).append(cu)
+            for key in [k for k, hs in members.items() if len(hs) == npos]:
+                for cu in holder.pop(key):
+                    room[cu] += 1
+                del members[key]
+                progressed = True
+            assert progressed, f"XCD {xcd}: {len(members)} channels wait for blocks that cannot start"
+        assert seated == len(all_seats(d)) // XCDS
 
 
 def test_a_small_launch_is_seated_in_the_order_of_arrival():
@@ -163,10 +277,15 @@ def test_a_small_launch_is_seated_in_the_order_of_arrival():
 def test_seat_arguments_are_checked():
     L = _lib.lib()
     d = op_for(**CASES[0])
-    none = [None] * 5
-    assert L.mint_ring_seat(d, 8, 0, 0, 0, *none) == _lib.ERR_ARG
-    assert L.mint_ring_seat(d, 0, -1, 0, 0, *none) == _lib.ERR_ARG
+    none = [None] * 3
+    state = (ctypes.c_uint64 * _lib.SEAT_STATE_WORDS)()
+    assert L.mint_ring_seat(d, 8, 0, 0, state, *none) == _lib.ERR_ARG
+    assert L.mint_ring_seat(d, 0, -1, 0, state, *none) == _lib.ERR_ARG
+    assert L.mint_ring_seat(d, 0, 0, 0, None, *none) == _lib.ERR_ARG
     spread = op_for(**{**CASES[0], "placement": _lib.PLACE_SPREAD, "cache_policy": 0})
-    assert L.mint_ring_seat(spread, 0, 0, 0, 0, *none) == _lib.ERR_ARG
-    # beyond a compute unit's share and beyond the leftover entries: nothing to do
-    assert L.mint_ring_seat(d, 0, 0, 1000, 1000, *none) == 0
+    assert L.mint_ring_seat(spread, 0, 0, 0, state, *none) == _lib.ERR_ARG
+    # one block more than the list has entries: nothing to do
+    per_xcd = L.mint_ring_grid_blocks(d) // XCDS
+    for i in range(per_xcd):
+        assert L.mint_ring_seat(d, 0, i % CUS, i // CUS, state, *none) == 1
+    assert L.mint_ring_seat(d, 0, 0, 1000, state, *none) == 0
