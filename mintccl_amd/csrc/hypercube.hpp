@@ -33,7 +33,6 @@
 
 namespace mint {
 
-enum : int { OP_HYPER_REDUCESCATTER = 10, OP_HYPER_ALLGATHER = 11 };
 constexpr int kHyperMaxDim = 3;      // 8 ranks
 
 __host__ __device__ __forceinline__ int hyper_dim(int world) {

@@ -42,7 +42,10 @@
 namespace mint {
 
 enum : int { OP_SENDRECV = 0, OP_BROADCAST = 1, OP_REDUCE = 2, OP_ALLGATHER = 3,
-             OP_REDUCESCATTER = 4, OP_ALLREDUCE = 5, OP_ALLTOALL = 6 };
+             OP_REDUCESCATTER = 4, OP_ALLREDUCE = 5, OP_ALLTOALL = 6,
+             // (walks of their own: tree.hpp, temporal.hpp, hypercube.hpp)
+             OP_TREE_BROADCAST = 7, OP_TREE_REDUCE = 8, OP_ALLGATHER_TEMPORAL = 9,
+             OP_HYPER_REDUCESCATTER = 10, OP_HYPER_ALLGATHER = 11 };
 enum : int { PROTO_LL128 = 0, PROTO_SIMPLE = 1 };
 enum : int { PLACE_SPREAD = 0, PLACE_LOCAL = 1 };
 
@@ -295,13 +298,18 @@ __host__ __device__ __forceinline__ int seat_claim(const SeatList& l, int wanted
 }
 // A list of at most one round (a small launch: no compute unit gets a second
 // block) is simply taken in the order in which the blocks reach one counter:
-// one atomic instead of three trips.  (Not so the longer lists of launches
-// whose position count does not divide the compute units anyway, like the 9 of
-// a reduce-scatter: taken in the order of arrival, the 8 x 256 MiB
-// reduce-scatter needs 8 % longer.)
+// one trip to the counter instead of three or four in a row.  So is the list
+// of a launch of fewer than kSeatByCuMinSteps steps, whose few microseconds
+// gain more from the shorter start than from a neat division of the positions
+// over the compute units (8 ranks, 1 - 4 MiB per rank: -1.5 us of 14 - 28; from
+// 17 steps on the copying collectives, whose origins want compute units of
+// their own, lose 20 % that way, and long reductions 5 - 8 %; a temporal
+// allgather runs its steps once per rank).
+constexpr uint32_t kSeatByCuMinSteps = 16;
 __host__ __device__ __forceinline__ bool seats_in_order_of_arrival(const RingArgs& a,
                                                                    const SeatList& l) {
-    return l.full == 0;
+    const uint32_t steps = a.op == OP_ALLGATHER_TEMPORAL ? a.steps * (uint32_t)a.world : a.steps;
+    return l.full == 0 || steps < kSeatByCuMinSteps;
 }
 // What entry y of XCD `xcd` is: pipeline, position, block of the group.
 __host__ __device__ __forceinline__ bool seat_of_entry(const RingArgs& a, int xcd, int y, int& p,

@@ -32,8 +32,6 @@
 
 namespace mint {
 
-enum : int { OP_ALLGATHER_TEMPORAL = 9 };
-
 template <int CPI>
 __device__ __forceinline__ void temporal_walk(const RingArgs& a, const int h, const int w) {
     constexpr int LDCP = Policy<CPI>::LD, STCP = Policy<CPI>::ST;

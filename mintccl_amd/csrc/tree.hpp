@@ -30,7 +30,6 @@
 
 namespace mint {
 
-enum : int { OP_TREE_BROADCAST = 7, OP_TREE_REDUCE = 8 };
 constexpr int kTreeArity = 2;
 
 __host__ __device__ __forceinline__ int tree_rank(const RingArgs& a, int h) {
