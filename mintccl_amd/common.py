@@ -226,8 +226,9 @@ def tuned_origin_cus(op: int, npos: int, channels: int, waves_per_block: int) ->
     broadcast, an allgather or an alltoall get to themselves; ``npos`` = positions of a
     pipeline, ``channels`` = thread blocks per position of the launch (the
     library ignores the number for small grids and other collectives).  A CU
-    keeps about 26 KB of loads in flight and a load from HBM takes 2.5 us
-    while the collective's stores saturate it, so the origins' natural share
+    keeps a bounded number of requests in flight (about 15 KB of loads) and a
+    load from HBM takes several times longer than usual while the
+    collective's stores keep HBM busy, so the origins' natural share
     of the CUs - one position in ``npos`` - delivers too little: measured
     best at 8 positions is 9 of 32 (allgather of 8 x 128 MiB 3.38 -> 2.57 ms,
     broadcast of 64 MiB 0.237 -> 0.171 ms), 2.25 times the natural share,
