@@ -121,8 +121,9 @@ typedef enum {
 /* Status block written by the ring kernel (device memory, 4 x uint64, zeroed
  * by the caller before launch).  word 0: 0 = OK, else 1 = a bounded wait ran
  * out; word 1: (pipeline << 32 | position << 16 | wave) of the first waiter
- * that gave up; word 2: step it waited for; word 3: abort flag polled by all
- * other waits.  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
+ * that gave up; word 2: step it waited for; word 3: low half = abort flag
+ * polled by all other waits, high half = number of launches that started
+ * with the flag already set (they give up at their first wait).  Error code 2: MINT_PLACE_LOCAL met an XCD number beyond 7; word 2
  * then holds that number.  Error code 3: MINT_PLACE_LOCAL, and a thread block
  * found every seat of its XCD taken or waited in vain for its compute unit's
  * number: the device did not deal an eighth of the grid to every XCD (blocks

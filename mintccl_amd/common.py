@@ -587,9 +587,11 @@ class VirtualComm:
                     "the device did not deal an eighth of the thread blocks to every XCD, so a "
                     "block of the local placement found no seat; outputs are unspecified - use "
                     "placement spread (and cache_policy 0) on this stream")
+            later = (st[3] >> 32) & 0xFFFFFFFF
             raise RingTimeout(
                 f"ring kernel wait ran out: pipeline {who >> 32}, position "
-                f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]} "
+                f"{(who >> 16) & 0xFFFF}, wave {who & 0xFFFF}, step {st[2]}; {later} later "
+                "launch(es) found the abort flag set and gave up "
                 "(outputs of every launch since the last check are unspecified)")
 
 

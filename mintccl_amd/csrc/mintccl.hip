@@ -727,6 +727,7 @@ int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, uint64
     uint64_t* const taken = state;
     uint64_t& tickets = state[kSeatWords];
     int y;
+    bool filled = false;
     if (seats_in_order_of_arrival(plan.args, list)) {
         // taken in the order of arrival at one counter per XCD
         y = tickets < (uint64_t)list.len ? (int)tickets : -1;
@@ -739,7 +740,7 @@ int mint_ring_seat(const mint_ring_op* op, int xcd, int cu_rank, int nth, uint64
                 taken[word] |= bits;
                 return before;
             },
-            [&]() { return (int)tickets++; });
+            [&]() { return (int)tickets++; }, filled);
     }
     int p = 0, h = 0, gw = 0;
     if (y < 0 || !seat_of_entry(plan.args, xcd, y, p, h, gw)) return 0;

@@ -126,8 +126,9 @@ __device__ __forceinline__ Role role_of(const RingArgs& a, int p, int h) {
 }
 
 // First wavefront that gives up records why (1 = a bounded wait ran out,
-// 2 = the local placement met an XCD number beyond 7) and who it was;
-// everybody else sees word 3.
+// 2 = the local placement met an XCD number beyond 7, 3 = no seat) and who
+// it was; everybody else sees word 3: its low half is the abort flag, its
+// high half counts the launches that started with the flag set.
 __device__ __forceinline__ void report_error(uint64_t* status, uint64_t code, int p, int h, int w,
                                              uint64_t detail) {
     if (lane_id() == 0) {
@@ -136,7 +137,8 @@ __device__ __forceinline__ void report_error(uint64_t* status, uint64_t code, in
             st64_agent(status + 1, ((uint64_t)p << 32) | ((uint64_t)h << 16) | (uint64_t)w);
             st64_agent(status + 2, detail);
         }
-        st64_agent(status + 3, 1ull);
+        __hip_atomic_fetch_or((MINT_GLOBAL unsigned long long*)(s + 3), 1ull, __ATOMIC_RELAXED,
+                              __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 __device__ __forceinline__ void report_timeout(uint64_t* status, int p, int h, int w,
@@ -145,6 +147,15 @@ __device__ __forceinline__ void report_timeout(uint64_t* status, int p, int h, i
 }
 __device__ __forceinline__ bool aborted(const uint64_t* status) {
     return __builtin_amdgcn_readfirstlane((uint32_t)ld64_agent(status + 3)) != 0u;
+}
+// One wavefront per launch: a launch that starts with the abort flag set (an
+// earlier launch on this status block gave up and the caller has not looked
+// yet) gives up at its first wait; count it, so that the caller learns how
+// many launches ran for nothing.
+__device__ __forceinline__ void count_launch_if_aborted(uint64_t* status, int wave_of_block) {
+    if (blockIdx.x == 0 && wave_of_block == 0 && lane_id() == 0 && aborted(status))
+        __hip_atomic_fetch_add((MINT_GLOBAL unsigned long long*)(status + 3), 1ull << 32,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Spin until the credit / head word at `word` carries this epoch and a count
@@ -228,7 +239,8 @@ __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int
 //                           23:0, j + 1 in bits 31:24 once it is known
 //   16384 + xcd * 128       per XCD, a line of its own: + 0 compute units
 //                           registered, + 8 tickets handed out, + 16 entries
-//                           claimed
+//                           claimed (a list taken in the order of arrival) or
+//                           words of the map that are full
 //   18432 + xcd * 128       per XCD, a line of its own: the map of taken
 //                           entries, 1024 bits
 // A line that blocks of several XCDs work on is slow (a counter per XCD in one
@@ -272,25 +284,38 @@ __host__ __device__ __forceinline__ int seat_wanted(const SeatList& l, int j, in
 // entry 0, and takes the first free entry from there upwards (round the list).
 // `fetch_or(word, bits)` sets bits in word `word` of the XCD's map of taken
 // entries and returns what the word held before; `draw()` hands out the next
-// ticket.  -1: no entry is free (more blocks than entries).
+// ticket.  -1: no entry is free (more blocks than entries).  `filled_a_word`
+// comes back true for the block whose claim set the last free entry of a word
+// of the map: exactly one block per word learns that.
 template <class FetchOr, class Draw>
 __host__ __device__ __forceinline__ int seat_claim(const SeatList& l, int wanted, FetchOr fetch_or,
-                                                   Draw draw) {
-    if (wanted >= 0 && !((fetch_or(wanted >> 6, 1ull << (wanted & 63)) >> (wanted & 63)) & 1ull))
-        return wanted;
+                                                   Draw draw, bool& filled_a_word) {
+    const int last_word = (l.len - 1) >> 6;
+    // bits of word `word` that stand for entries of the list
+    auto entries_of = [&](int word) {
+        return word == last_word && (l.len & 63) ? (1ull << (l.len & 63)) - 1ull : ~0ull;
+    };
+    filled_a_word = false;
+    if (wanted >= 0) {
+        const uint64_t bit = 1ull << (wanted & 63), before = fetch_or(wanted >> 6, bit);
+        if (!(before & bit)) {
+            filled_a_word = (before | bit) == entries_of(wanted >> 6);
+            return wanted;
+        }
+    }
     const int t = draw();
     int e = t < l.rest ? l.full * kCusPerXcd + t : 0;
-    const int last_word = (l.len - 1) >> 6;
     // (every miss means that another block took an entry, so len looks and a
     // walk over the words suffice)
     for (int looks = 0; looks < l.len + 2 * kSeatWords; ++looks) {
         const int word = e >> 6, bit = e & 63;
         const uint64_t before = fetch_or(word, 1ull << bit);
-        if (!((before >> bit) & 1ull)) return e;
+        if (!((before >> bit) & 1ull)) {
+            filled_a_word = (before | (1ull << bit)) == entries_of(word);
+            return e;
+        }
         // the lowest entry of this word above e that was free a moment ago
-        uint64_t free_above = ~before & ~((2ull << bit) - 1ull);
-        if (bit == 63) free_above = 0;
-        if (word == last_word && (l.len & 63)) free_above &= (1ull << (l.len & 63)) - 1ull;
+        const uint64_t free_above = ~before & ~((2ull << bit) - 1ull) & entries_of(word);
         if (free_above) e = word * 64 + __builtin_ctzll(free_above);
         else e = word < last_word ? (word + 1) * 64 : 0;
     }
@@ -379,7 +404,7 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& la
     const SeatList list = seat_list(a, (int)gridDim.x);
     uint64_t* const line = ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride);
     int y;
-    uint32_t claimed;
+    uint32_t claimed = 0;
     if (seats_in_order_of_arrival(a, list)) {
         claimed = (uint32_t)ticket_add(line + 2, 1ull);
         y = (int)claimed < list.len ? (int)claimed : -1;
@@ -410,6 +435,7 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& la
             jfield &= 0xFFu;
         }
         uint64_t* const taken = ticket_word(a, kTicketTaken + (uint32_t)xcd * kTicketXcdStride);
+        bool filled = false;
         y = seat_claim(
             list, seat_wanted(list, (int)jfield - 1, (int)nth),
             [&](int word, uint64_t bits) {
@@ -417,12 +443,17 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& la
                                                        (unsigned long long)bits, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT);
             },
-            [&]() { return (int)ticket_add(line + 1, 1ull); });
+            [&]() { return (int)ticket_add(line + 1, 1ull); }, filled);
         if (y < 0) {
             report_error(a.status, 3, 0, 0, 0, (uint64_t)cu);
             return -1;
         }
-        claimed = (uint32_t)ticket_add(line + 2, 1ull);
+        // The block that fills the last word of the map has claimed the last
+        // entry of the list (words are counted as they fill up: one more trip
+        // for 4 - 16 blocks per XCD instead of one for every block).
+        const uint32_t words = (uint32_t)((list.len + 63) >> 6);
+        last = filled && (uint32_t)ticket_add(line + 2, 1ull) + 1u == words;
+        return y;
     }
     if (y < 0) return -1;
     // the block that claims the last entry of its XCD's list clears up
@@ -451,6 +482,7 @@ __device__ __forceinline__ Seat take_seat(const RingArgs& a, int wpb, int wib, i
     // the whole struct in scratch memory)
     int p = 0, h = 0, gw = 0;
     bool seated = true;
+    count_launch_if_aborted(a.status, wave_of_block);
     if (a.placement == PLACE_LOCAL) {
         if (wave_of_block == 0 && lane_id() == 0) {       // one lane: the counters count blocks
             int xcd = 0;
@@ -1295,8 +1327,6 @@ __global__ void __launch_bounds__(512) ring_kernel(const RingArgs a) {
     // scratch memory)
     const int p = st.p, h = st.h, w = st.w;
     const Role role = role_of(a, p, h);
-    // a position that writes a caller's buffer first makes sure that every
-    // (channel, position) of the launch has a thread block
     walk_as<PROTO, DT, CPI, U, false>(a, p, h, w, role);
 }
 

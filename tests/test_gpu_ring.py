@@ -624,7 +624,16 @@ def test_a_lost_producer_times_out_instead_of_hanging(dev):
                      {r: bufs[r].data_ptr() for r in range(1, world)}, [0, 1, 2, 3, 0],
                      root=0, skip_origin=True)
     comm.launch(d)
-    with pytest.raises(RingTimeout):
+    # two more launches queued behind the one that gives up: they find the abort
+    # flag set, give up at their first wait and are counted
+    full = comm.make_op(_lib.OP_BROADCAST, _lib.BYTES, n * 2, {0: bufs[0].data_ptr()},
+                        {r: bufs[r].data_ptr() for r in range(1, world)}, [0, 1, 2, 3, 0], root=0)
+    comm.launch(full)
+    comm.launch(full)
+    torch.cuda.synchronize(dev)
+    st = comm.status.cpu().tolist()
+    assert st[0] == 1 and (st[3] & 0xFFFFFFFF) == 1 and (st[3] >> 32) == 2
+    with pytest.raises(RingTimeout, match="2 later launch"):
         comm.check()
     # the communicator is usable afterwards
     host = [normal(n, r) for r in range(world)]
