@@ -266,6 +266,26 @@ def test_a_partly_resident_grid_fills_whole_channels(case, cus, per_cu):
         assert seated == len(all_seats(d)) // XCDS
 
 
+def test_random_deals_seat_every_block_exactly_once():
+    """Any multiset of compute units, in any order: as many blocks as entries
+    means every seat is taken exactly once (25 random launches per case, every XCD its own deal, from one
+    compute unit taking everything to 60 compute units sharing)."""
+    rng = random.Random(2024)
+    for kw in (CASES[0], CASES[1], CASES[3], CASES[7]):
+        d = op_for(**kw)
+        want = all_seats(d)
+        per_xcd = L_grid(d) // XCDS
+
+        def deal(xcd, count):
+            ncu = rng.choice((1, 2, 3, 7, 16, 31, 32, 33, 40, 60))
+            weights = [rng.random() ** 3 + 0.01 for _ in range(ncu)]
+            return rng.choices(range(ncu), weights=weights, k=count)
+        for _ in range(25):
+            taken = seats_for(d, deal)
+            assert len(taken) == len(set(taken)) and set(taken) == want
+        assert per_xcd == len(want) // XCDS or kw.get("origin_cus")
+
+
 def test_a_small_launch_is_seated_in_the_order_of_arrival():
     # at most one round (32 entries per XCD): one counter per XCD hands out the
     # entries, so only the XCDs' shares have to be right
