@@ -21,7 +21,8 @@ are what they are measured against.
 ``python -m mintccl_amd.yardsticks --counters [waves]`` launches, twice each
 and for one wavefront count (default 4032, the headline launch's), the kernels
 a counter run compares: the headline reduce-scatter itself, the mix at 1 - 4
-steps in flight, its parts alone, and the read-only pass; meant to run under
+steps in flight, its parts alone, the mix of a copying position, and the
+read-only pass; meant to run under
 ``rocprofv3 --pmc``.  No counterpart in the reference.
 """
 from __future__ import annotations
@@ -97,6 +98,10 @@ def counters(dev: torch.device, waves: int) -> int:
         primitive.step_mix_deep(rows, staging, waves, steps_for(waves, 3), 6, 3)
         primitive.step_mix_deep(rows, staging, waves, steps_for(waves, 3), 2, 3)
         primitive.step_mix_deep(rows, staging, waves, steps_for(waves, 3), 4, 3)
+        # what a copying position does: the streaming store to HBM alone, and
+        # with the staging load and store around it
+        primitive.step_mix(rows, staging, waves, steps_for(waves, 0), 16)
+        primitive.step_mix(rows, staging, waves, steps_for(waves, 0), 22)
     torch.cuda.synchronize()
     print(json.dumps({"counters": "launched", "wavefronts": waves}), flush=True)
     return 0
