@@ -135,6 +135,36 @@ def test_static_launch_of_the_tree_and_the_temporal_schedule(dev, lib):
         assert np.array_equal(as_bytes(g[r]), want[r]), r
 
 
+@pytest.mark.gpu
+def test_static_launch_over_the_hypercube(dev, lib):
+    """Recursive halving and doubling through the static array (seven shares
+    per slot), under the local placement too."""
+    status = torch.zeros(4, dtype=torch.int64, device=dev)
+    n = 20011
+    for placement, cache in ((_lib.PLACE_SPREAD, 0), (_lib.PLACE_LOCAL, 2)):
+        host = rank_rows(WORLD, n, "f16", seed0=90)
+        bufs = [h.to(dev) for h in host]
+        d = descriptor(_lib.OP_HYPERCUBE_REDUCESCATTER, _lib.F16, _lib.PROTO_LL128, n * 2,
+                       [t.data_ptr() for t in bufs], status, slot_bytes=7 * 16 * 1024, nslots=3,
+                       waves=16)
+        d.row_stride = n * 2
+        d.placement, d.cache_policy = placement, cache
+        launch_static(lib, d)
+        assert ok(status)
+        want = ring.hypercube_reducescatter([as_bytes(h) for h in host], "f16")
+        for r in range(WORLD):
+            assert np.array_equal(as_bytes(bufs[r]), want[r]), r
+        d = descriptor(_lib.OP_HYPERCUBE_ALLGATHER, _lib.BYTES, _lib.PROTO_LL128, n * 2,
+                       [t.data_ptr() for t in bufs], status, slot_bytes=7 * 16 * 1024, nslots=3,
+                       waves=16)
+        d.row_stride = n * 2
+        d.placement, d.cache_policy = placement, cache
+        launch_static(lib, d)
+        assert ok(status)
+        for r, w in enumerate(ring.allgather(want)):
+            assert np.array_equal(as_bytes(bufs[r]), w), r
+
+
 def forged_simple_broadcast(lib, dev, status):
     """A Simple broadcast through the static array whose payload is what an
     LL128 launch of any epoch would take for its sector tags."""
