@@ -234,11 +234,12 @@ __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int
 // units masked off - the blocks that are there have to fill whole channels,
 // lowest first, or they wait for blocks that cannot start.)
 //
-// The counters (64-bit words in device memory, zero between launches):
+// The counters (64-bit words in device memory, zero at first; between
+// launches zero again but for the compute units' ranks):
 //   xcd * 2048 + cu * 8     per compute unit: blocks that have arrived in bits
-//                           23:0, j + 1 in bits 31:24 once it is known
+//                           23:0, j + 1 in bits 31:24 once it is known (kept)
 //   16384 + xcd * 128       per XCD, a line of its own: + 0 compute units
-//                           registered, + 8 tickets handed out, + 16 entries
+//                           registered (kept), + 8 tickets handed out, + 16 entries
 //                           claimed (a list taken in the order of arrival) or
 //                           words of the map that are full
 //   18432 + xcd * 128       per XCD, a line of its own: the map of taken
@@ -247,7 +248,7 @@ __device__ __forceinline__ int seat_wave(const RingArgs& a, int gw, int wpb, int
 // line: 40 - 60 us for 160 blocks per XCD; in lines of their own: 6 us), hence
 // the spacing.  The block that claims the last entry of its XCD's list puts
 // that XCD's counters back to zero, so a launch finds them as the launch
-// before left them - zero - and the common path is one atomic per counter
+// before left them and the common path is one atomic per counter
 // (with the launch epoch in every word instead, every block of a launch found
 // a stale word first and went through a compare-and-swap: three more trips).
 // Nothing waits for the whole grid to be seated: a launch whose blocks are
@@ -416,7 +417,8 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& la
         const uint32_t nth = before & 0xFFFFFFu;
         uint32_t jfield = before >> 24;
         if (before == 0u) {
-            // first block of this compute unit: register the unit, publish its j
+            // first block this compute unit ever ran on this staging: register
+            // the unit, publish its j (which stays: later launches find it)
             jfield = (uint32_t)ticket_add(line, 1ull) + 1u;
             if (jfield > 0xFFu) jfield = 0xFFu;
             __hip_atomic_fetch_or((MINT_GLOBAL unsigned long long*)word,
@@ -460,15 +462,23 @@ __device__ __forceinline__ int claim_entry(const RingArgs& a, int& xcd, bool& la
     last = claimed + 1u == (uint32_t)list.len;
     return y;
 }
-// Puts the counters of XCD `xcd` back to zero (the thread block that claimed
-// the last entry of the XCD's list; every other claim of the launch on this
-// XCD has been counted by then).
+// Puts the counters of XCD `xcd` back for the next launch (the thread block
+// that claimed the last entry of the XCD's list; every other claim of the
+// launch on this XCD has been counted by then).  What stays is the compute
+// units' ranks - the j of every unit that has registered and the count of
+// those - so that from the second launch on a block reads its unit's j from
+// the word it counts itself on, instead of registering the unit again (two
+// trips fewer at the start of every launch, and nobody waits for a j).
 __device__ __forceinline__ void reset_tickets(const RingArgs& a, int xcd) {
-    for (uint32_t i = threadIdx.x; i < 256u + 3u + (uint32_t)kSeatWords; i += blockDim.x) {
+    for (uint32_t i = threadIdx.x; i < 256u + 2u + (uint32_t)kSeatWords; i += blockDim.x) {
+        if (i < 256u) {
+            __hip_atomic_fetch_and((MINT_GLOBAL unsigned long long*)ticket_word(a, (uint32_t)xcd * 2048u + i * 8u),
+                                   0xFF000000ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
+        }
         uint64_t* const w =
-            i < 256u ? ticket_word(a, (uint32_t)xcd * 2048u + i * 8u)
-            : i < 259u ? ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride) + (i - 256u)
-                       : ticket_word(a, kTicketTaken + (uint32_t)xcd * kTicketXcdStride) + (i - 259u);
+            i < 258u ? ticket_word(a, kTicketXcdLine + (uint32_t)xcd * kTicketXcdStride) + (i - 255u)
+                     : ticket_word(a, kTicketTaken + (uint32_t)xcd * kTicketXcdStride) + (i - 258u);
         __hip_atomic_store((MINT_GLOBAL unsigned long long*)w, 0ull, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
