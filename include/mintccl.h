@@ -206,8 +206,8 @@ typedef struct {
                               hold nothing but origins (the positions that
                               read the caller's rows from HBM): SENDRECV,
                               BROADCAST, TREE_BROADCAST, ALLGATHER(_TEMPORAL) and ALLTOALL under MINT_PLACE_LOCAL
-                              with at least 64 thread blocks per position,
-                              below 32; ignored elsewhere, and
+                              with at least 64 thread blocks per position
+                              and 16 steps, below 32; ignored elsewhere, and
                               where the larger grid it needs (blocks with
                               nothing to do fill the rounds) would not be
                               resident.  A matter of speed only: a compute

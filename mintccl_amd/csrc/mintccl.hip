@@ -296,7 +296,11 @@ int make_plan(const mint_ring_op* op, Plan* plan, bool for_launch = false,
         const int origin_cus = (int)op->origin_cus;
         if (origin_cus >= kCusPerXcd || op->reserved1) return MINT_ERR_ARG;
         plan->blocks_plain = plan->blocks;
+        // (not for a launch so short that its seats are taken in the order of
+        // arrival: there the list's order does not decide what a compute unit holds)
+        const uint32_t walk_steps = temporal ? a.steps * (uint32_t)op->world : a.steps;
         if (op->placement == MINT_PLACE_LOCAL && origin_cus > 0 && npos >= 2 && groups >= 8 &&
+            walk_steps >= kSeatByCuMinSteps &&
             (op->op == MINT_OP_BROADCAST || op->op == MINT_OP_ALLGATHER ||
              op->op == MINT_OP_SENDRECV || op->op == MINT_OP_ALLTOALL || temporal ||
              op->op == MINT_OP_TREE_BROADCAST)) {

@@ -186,10 +186,13 @@ def test_compute_units_set_apart_for_origins_grow_the_grid():
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **big)) == 8 * 32 * 5
     assert L.mint_ring_grid_blocks(make_op(origin_cus=4, **big)) == 8 * 32 * 4     # the natural share
     assert L.mint_ring_grid_blocks(make_op(origin_cus=16, **big)) == 8 * 32 * 7
-    bc = dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, cache_policy=2,
+    bc = dict(op=_lib.OP_BROADCAST, dtype=_lib.BYTES, placement=1, cache_policy=2, count_bytes=64 << 20,
               slot_bytes=512 << 10, nslots=3, waves_per_channel_group=512)
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **bc)) == 8 * 32 * 5
-    # ignored: small grids, the spread placement, other collectives
+    # ignored: launches of fewer than 16 steps (their seats are taken in the order of
+    # arrival), small grids, the spread placement, other collectives
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **dict(bc, count_bytes=4 << 20))) == 8 * 8 * 16
+    assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **dict(bc, count_bytes=8 << 20))) == 8 * 32 * 5
     small = dict(big, waves_per_channel_group=16, slot_bytes=128 << 10)
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **small)) == 8 * 8 * 4
     assert L.mint_ring_grid_blocks(make_op(origin_cus=9, **dict(big, placement=0, cache_policy=0))) == 8 * 8 * 16
@@ -197,7 +200,8 @@ def test_compute_units_set_apart_for_origins_grow_the_grid():
     # a sendrecv over one hop: 64 channels per XCD, 20 CUs for the origins (4 rounds), 12 for
     # the destinations (6 rounds)
     sr = make_op(origin_cus=20, op=_lib.OP_SENDRECV, dtype=_lib.BYTES, placement=1, cache_policy=2,
-                 route_len=2, slot_bytes=1536 << 10, nslots=4, waves_per_channel_group=1536)
+                 count_bytes=256 << 20, route_len=2, slot_bytes=1536 << 10, nslots=4,
+                 waves_per_channel_group=1536)
     sr.ring[0], sr.ring[1] = 0, 1
     assert L.mint_ring_grid_blocks(sr) == 8 * 32 * 4
     sr.threads_per_block = 128
