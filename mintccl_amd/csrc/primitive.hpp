@@ -161,22 +161,24 @@ __device__ __forceinline__ void st64_stream(void* p, u32x2 v) {
 
 // ---- element addition: one IEEE round-to-nearest-even per call ------------
 // f16: v_pk_add_f16 (subnormals kept; the kernel is compiled without
-// flush-to-zero).  bf16: widen, one binary32 add, round to nearest even on the
-// bit pattern, NaN -> 0x7FC0.  f32: v_add_f32.
+// flush-to-zero).  bf16: widen, one binary32 add, round to nearest even
+// (v_cvt_pk_bf16_f32), NaN -> 0x7FC0.  f32: v_add_f32.
 __device__ __forceinline__ uint32_t add_f16x2(uint32_t a, uint32_t b) {
     f16x2 x = __builtin_bit_cast(f16x2, a), y = __builtin_bit_cast(f16x2, b);
     return __builtin_bit_cast(uint32_t, x + y);
 }
-__device__ __forceinline__ uint32_t bf16_round(float s) {
-    uint32_t bits = __builtin_bit_cast(uint32_t, s);
-    uint32_t r = (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
-    return (s != s) ? 0x7FC0u : r;
-}
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
-    float lo = __builtin_bit_cast(float, a << 16) + __builtin_bit_cast(float, b << 16);
-    float hi = __builtin_bit_cast(float, a & 0xFFFF0000u) +
-               __builtin_bit_cast(float, b & 0xFFFF0000u);
-    return bf16_round(lo) | (bf16_round(hi) << 16);
+    f32x2 s;
+    s.x = __builtin_bit_cast(float, a << 16) + __builtin_bit_cast(float, b << 16);
+    s.y = __builtin_bit_cast(float, a & 0xFFFF0000u) + __builtin_bit_cast(float, b & 0xFFFF0000u);
+    // both sums to bf16 in one instruction (v_cvt_pk_bf16_f32: round to nearest
+    // even); a NaN becomes the canonical one
+    uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(s, bf16x2));
+    if (s.x != s.x) bits = (bits & 0xFFFF0000u) | 0x7FC0u;
+    if (s.y != s.y) bits = (bits & 0x0000FFFFu) | 0x7FC00000u;
+    return bits;
 }
 __device__ __forceinline__ uint32_t add_f32(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t,
