@@ -398,6 +398,40 @@ def test_local_placement_on_a_stream_confined_to_half_of_the_compute_units(dev):
 
 
 @pytest.mark.gpu
+def test_local_placement_beside_another_streams_kernels(dev):
+    """A collective under the local placement while matrix products of another
+    stream hold part of the compute units: the thread blocks land on whatever
+    units have room, in whatever numbers, and still find their seats."""
+    from mintccl_amd import _lib
+    from mintccl_amd.allgather import allgather
+    from mintccl_amd.common import VirtualComm
+    from mintccl_amd.reducescatter import reducescatter
+    world, n = 8, 524309
+    comm = VirtualComm(world_size=world, device=dev, spin_budget=4000000)
+    assert comm.placement == _lib.PLACE_LOCAL
+    host = rank_rows(world, n, "f16", 8200)
+    want = ring.reducescatter([as_bytes(h) for h in host], "f16")
+    gathered = ring.allgather(want)
+    bufs = [h.to(dev) for h in host]
+    a = torch.randn(8192, 8192, device=dev, dtype=torch.float16)
+    other = torch.cuda.Stream(device=dev)
+    for _ in range(4):
+        for b, h in zip(bufs, host):
+            b.copy_(h)
+        torch.cuda.synchronize(dev)
+        with torch.cuda.stream(other):
+            for _ in range(6):
+                a @ a
+        comm.run(lambda r: reducescatter(bufs[r], comm))
+        assert comm.last_grid >= 8 * 64
+        comm.run(lambda r: allgather(bufs[r], comm))
+        comm.check()
+        other.synchronize()
+        for b, w in zip(bufs, gathered):
+            assert np.array_equal(as_bytes(b), w)
+
+
+@pytest.mark.gpu
 def test_captured_ll128_launch_replayed_after_an_eager_simple_launch(dev):
     """A communicator with its epoch in device memory: an LL128 allgather is
     captured while the launch before it was LL128 too; between the replays an
