@@ -112,7 +112,9 @@ class Timer:
 # Tuned geometry for MI355X (measured), one 1 KiB block per wave-channel per
 # step.  3 slots of 512 KiB and 4608 wavefronts, with these exceptions:
 # reducescatter 3 slots of 448 KiB, 56 wave-channels per (row, hop) instead of
-# 64 (1.5 - 2 % faster); an LL128 sendrecv over one hop 4 slots of 1.5 MiB;
+# 64 (1.5 - 2 % faster: 4032 wavefronts are at most 16 on a compute unit, and
+# the device serves the collectives' access mix a fifth slower with 18), and
+# the ring reduce likewise 448 wave-channels per position (-3 %); an LL128 sendrecv over one hop 4 slots of 1.5 MiB;
 # alltoall 6 slots and 2560 wavefronts in all under LL128, 2 slots and 5760
 # under Simple.  A slot may grow to TUNED_SLOT_BUDGET bytes when there are few
 # hops.  Sendrecv, broadcast, allgather and alltoall set compute units apart
@@ -203,7 +205,8 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         npos = (npos + 1) // 2    # `pipes` already counts both phases
     # slots sized per 8 receiving ranks keep the staging of an XCD's channels
     # (slots x receivers / 8) well inside its 4 MiB of L2
-    per8 = TUNED_SLOT_BLOCKS_REDUCESCATTER if op == _lib.OP_REDUCESCATTER else TUNED_SLOT_BLOCKS
+    per8 = (TUNED_SLOT_BLOCKS_REDUCESCATTER if op in (_lib.OP_REDUCESCATTER, _lib.OP_REDUCE)
+            else TUNED_SLOT_BLOCKS)
     total = TUNED_TOTAL_WAVES
     if fetcher_waves:
         # every thread block carries one more wavefront (it streams own rows
