@@ -188,10 +188,12 @@ def tuned_geometry(op: int, world: int, route_len: int, threads_per_block: int,
         return fit(shares, max_nslots, waves, granule)
     if op in (_lib.OP_HYPERCUBE_REDUCESCATTER, _lib.OP_HYPERCUBE_ALLGATHER):
         # world rows x world nodes, one wavefront per (row, node, wave-channel);
-        # a rank's slot has a share per stream it receives: world - 1
+        # a rank's slot has a share per stream it receives: world - 1.  4096
+        # wavefronts are 16 on every compute unit (with 4608 an 8 x 64 MiB
+        # allgather takes 10 % longer)
         granule = wpb
         waves = max(granule, min(TUNED_SLOT_BUDGET // 1024 // max(1, world - 1),
-                                 TUNED_TOTAL_WAVES // (world * world)) // granule * granule)
+                                 4096 // (world * world)) // granule * granule)
         return fit(max(1, world - 1), max_nslots, waves, granule)
     pipes = world if op in (_lib.OP_ALLGATHER, _lib.OP_REDUCESCATTER, _lib.OP_ALLREDUCE) else 1
     real_pipes = pipes

@@ -132,8 +132,8 @@ CASES = [
     dict(op=_lib.OP_ALLREDUCE, count_bytes=16 << 20, slot_bytes=16 * 24 << 10, nslots=3,
          waves_per_channel_group=24, threads_per_block=192, **LOCAL),
     # a hypercube: 8 rows x 8 corners
-    dict(op=_lib.OP_HYPERCUBE_REDUCESCATTER, count_bytes=8 << 20, slot_bytes=7 * 72 << 10, nslots=3,
-         waves_per_channel_group=72, threads_per_block=256, **LOCAL),
+    dict(op=_lib.OP_HYPERCUBE_REDUCESCATTER, count_bytes=8 << 20, slot_bytes=7 * 64 << 10, nslots=3,
+         waves_per_channel_group=64, threads_per_block=256, **LOCAL),
 ]
 
 
