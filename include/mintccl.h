@@ -218,8 +218,9 @@ typedef struct {
 } mint_ring_op;
 
 /* 100 * major + minor of this interface: 102 = mint_build_flags, mint_static_init,
- * mint_step_mix_deep, mint_ring_seat; mint_epoch_advance takes the protocol;
- * every rank's staging grew by the seat tickets (101 = mint_ring_op with origin_cus).  A binding checks it against the
+ * mint_step_mix_deep, mint_ring_seat, MINT_OP_HYPERCUBE_*; mint_epoch_advance takes
+ * the protocol; every rank's staging grew by the seat counters; status word 3 counts
+ * launches that started aborted (101 = mint_ring_op with origin_cus).  A binding checks it against the
  * version it was written for before it passes a descriptor. */
 int mint_version(void);
 /* What the library was compiled with, as bits.  A product build returns 0.

@@ -26,8 +26,8 @@ static __device__ __align__(256) unsigned char scratch[MINT_STATIC_SCRATCH_BYTES
 namespace {
 
 constexpr int kVersion = 102;   // 0.1.2: mint_build_flags, mint_static_init, mint_step_mix_deep,
-                                // mint_ring_seat; mint_epoch_advance takes the protocol; staging
-                                // grew by the seat tickets
+                                // mint_ring_seat, the hypercube ops; mint_epoch_advance takes the
+                                // protocol; staging grew by the seat counters
 // What this library was compiled with (mint_build_flags).
 constexpr int kBuildFlags = 0
 #ifdef MINT_RING_STATS
