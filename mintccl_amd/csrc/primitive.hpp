@@ -64,6 +64,16 @@ template <int CP>
 __device__ __forceinline__ void st128(const Window& w, uint32_t off, u32x4 v) {
     __builtin_amdgcn_raw_buffer_store_b128(v, w.rsrc, (int)off, 0, CP);
 }
+// A load with a wave-uniform part of the offset in a scalar register (the
+// instruction adds it): what changes from step to step costs no vector add.
+// Loads only.  A 128-bit store with its offset in a scalar register was seen
+// to pick up the next vector instruction's write to its first data register
+// (word 0 of lanes 12 - 15 of every 16, now and then): the compiler leaves no
+// gap after such a store, which it does after one with a constant offset.
+template <int CP>
+__device__ __forceinline__ u32x4 ld128(const Window& w, uint32_t off, uint32_t uniform_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(w.rsrc, (int)off, (int)uniform_off, CP);
+}
 template <int CP>
 __device__ __forceinline__ u32x2 ld64(const Window& w, uint32_t off) {
     return __builtin_amdgcn_raw_buffer_load_b64(w.rsrc, (int)off, 0, CP);

@@ -1126,6 +1126,124 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         }
       }
     }
+    // ---- whole steps of the adding collectives ---------------------------------
+    // The same step as run_group's - credit word, polls, fetch of the next
+    // step's own rows, tags, credit post, add, save / send - with everything
+    // that does not change from step to step taken out of it: a CU has one
+    // scalar unit for its sixteen wavefronts, and the general group above
+    // spends 76 scalar instructions and 9 branches per step on bookkeeping
+    // (which group of the step, which blocks are valid, what the next group
+    // looks like).  The polls' staging offsets ride in the scalar offset of the
+    // buffer instruction, the row pointer and the tag advance by constants.
+    // Nothing is issued conditionally except the credit load (fetch addresses
+    // are clamped into the row), so every wait leaves exactly the fetch ahead
+    // in flight.  Steps that are not whole, and a library built for wait
+    // accounting, take the general path.
+    if constexpr (PROTO == PROTO_LL128 && DT != DT_BYTES && !LDSF) {
+      if (!timing && K == (uint32_t)U && ngroups) {
+        const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
+        uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
+        if (whole_steps > a.steps) whole_steps = a.steps;
+        if (whole_steps) {
+            u32x4 vv[2][U];
+            uint32_t step = 0, slot = 0, slot_off = 0;
+            uint32_t tag = (epoch << 20) | 1u;
+            int32_t need = 1 - (int32_t)a.nslots;            // credits step `step` needs, if positive
+            const uint32_t recv_v = share_recv * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
+            const uint32_t send_v = share_send * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
+            const uint32_t last_full = nfull - 1u;
+            constexpr uint64_t kDataLanes = 0x7777777777777777ull;    // every lane but the fourth of a sector
+            uint32_t g0 = (uint32_t)w;                      // block u = 0 of the step in hand
+            uint64_t cw = 0;
+            auto fetch_step = [&](uint32_t first, u32x4 (&x)[U]) MINT_INLINE_LAMBDA {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t g = first + (uint32_t)u * W;
+                    g = g < last_full ? g : last_full;       // beyond the whole blocks: any valid address
+                    x[u] = ll_fetch_raw(in_row, row_bytes, g, true, m);
+                }
+            };
+            auto give_up = [&]() MINT_INLINE_LAMBDA {
+                report_timeout(a.status, p, h, w, step);
+                __builtin_amdgcn_endpgm();
+            };
+            if (role.load) fetch_step(g0, vv[0]);
+            auto lean_step = [&](auto phase) MINT_INLINE_LAMBDA {
+                constexpr int B = decltype(phase)::value, B1 = B ^ 1;
+                u32x4 r[U];
+                // wait_ll128 (protocol.py:161-180): asked for ahead of the polls, looked at after them
+                const bool ask = role.send && (int32_t)credits_seen < need;
+                if (ask) cw = ld64_agent(nxt_tail);
+                if (role.recv) {
+                    compiler_fence();
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        r[u] = ld128<LDCP>(own, recv_v + (uint32_t)u * W * kBlockMsg, slot_off);
+                }
+                compiler_fence();
+                if (role.load) fetch_step(g0 + a.step_blocks, vv[B1]);
+                compiler_fence();
+                if (role.recv) {
+                    // recv_ll128 (protocol.py:102-130)
+                    uint32_t pending = 0;
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        if ((__ballot(r[u].w == tag) | kDataLanes) != ~0ull) pending |= 1u << u;
+                    for (uint32_t spins = 0; pending; ++spins) {
+                        if (spins >= a.spin_budget || ((spins & 63u) == 63u && aborted(a.status)))
+                            give_up();
+                        __builtin_amdgcn_s_sleep(1);
+                        compiler_fence();
+#pragma unroll
+                        for (int u = 0; u < U; ++u) {
+                            if (!(pending & (1u << u))) continue;
+                            r[u] = ld128<LDCP>(own, recv_v + (uint32_t)u * W * kBlockMsg, slot_off);
+                            if ((__ballot(r[u].w == tag) | kDataLanes) == ~0ull)
+                                pending &= ~(1u << u);
+                        }
+                    }
+                    // post_ll128 (protocol.py:183-189): the step is in registers,
+                    // the slot is free; every lane stores the same word
+                    if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1u));
+                    else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1u));
+                }
+                asm volatile("" : "+v"(cw));
+                if (ask) {
+                    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(cw >> 32));
+                    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)cw);
+                    if (hi == epoch && (int32_t)lo >= need) credits_seen = lo;
+                    else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
+                                         a.status))
+                        give_up();
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    u32x4 x = vv[B][u];
+                    if (role.load) x = ll_arrange(x, true, m);
+                    if (role.recv) x = role.reduce ? ll_comp<DT>(x, r[u]) : r[u];
+                    if (role.save) ll_save_raw(out_row, row_bytes, g0 + (uint32_t)u * W, true, m, x);
+                    if (role.send) {
+                        if (m.flag_lane) x.w = tag;
+                        st128<STCP>(nxt, send_v + (uint32_t)u * W * kBlockMsg + slot_off, x);
+                    }
+                }
+                ++step; ++tag; ++need;
+                g0 += a.step_blocks;
+                slot = slot + 1 == a.nslots ? 0 : slot + 1;
+                slot_off = slot ? slot_off + a.slot_bytes : 0;
+            };
+            while (step < whole_steps) {
+                lean_step(std::integral_constant<int, 0>{});
+                if (step >= whole_steps) break;
+                lean_step(std::integral_constant<int, 1>{});
+            }
+            // what is left (a ragged or partly filled last step) starts afresh
+            q.step = step; q.slot = slot; q.k0 = 0;
+            q.fill(geom);
+            n = step;
+        }
+      }
+    }
     if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
       if (!origin_done && K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
