@@ -1146,9 +1146,15 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         if (whole_steps > a.steps) whole_steps = a.steps;
         if (whole_steps) {
             u32x4 vv[2][U];
-            uint32_t step = 0, slot = 0, slot_off = 0;
+            // What moves from step to step: the tag, the credits the step needs
+            // (positive from step nslots on), the first block, the slot's offset.
+            uint32_t slot_off = 0;
             uint32_t tag = (epoch << 20) | 1u;
-            int32_t need = 1 - (int32_t)a.nslots;            // credits step `step` needs, if positive
+            const uint32_t end_tag = tag + whole_steps;
+            int32_t need = 1 - (int32_t)a.nslots;
+            // the same as a 64-bit word to compare the credit word with, kept in
+            // vector registers (a CU has one scalar unit and sixty-four vector lanes)
+            uint64_t need_word = flag_hi + (uint64_t)(int64_t)need;
             const uint32_t recv_v = share_recv * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t send_v = share_send * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t last_full = nfull - 1u;
@@ -1164,16 +1170,14 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 }
             };
             auto give_up = [&]() MINT_INLINE_LAMBDA {
-                report_timeout(a.status, p, h, w, step);
+                report_timeout(a.status, p, h, w, (uint32_t)(need + (int32_t)a.nslots) - 1u);
                 __builtin_amdgcn_endpgm();
             };
-            if (role.load) fetch_step(g0, vv[0]);
             auto lean_step = [&](auto phase) MINT_INLINE_LAMBDA {
                 constexpr int B = decltype(phase)::value, B1 = B ^ 1;
                 u32x4 r[U];
                 // wait_ll128 (protocol.py:161-180): asked for ahead of the polls, looked at after them
-                const bool ask = role.send && (int32_t)credits_seen < need;
-                if (ask) cw = ld64_agent(nxt_tail);
+                if (role.send && (int32_t)credits_seen < need) cw = ld64_agent(nxt_tail);
                 if (role.recv) {
                     compiler_fence();
 #pragma unroll
@@ -1204,14 +1208,16 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     }
                     // post_ll128 (protocol.py:183-189): the step is in registers,
                     // the slot is free; every lane stores the same word
-                    if (STCP == CP_NONE) st64_local(own_tail, flag_hi | (uint64_t)(step + 1u));
-                    else st64_agent(own_tail, flag_hi | (uint64_t)(step + 1u));
+                    const uint64_t posted = flag_hi | (uint64_t)(uint32_t)(need + (int32_t)a.nslots);
+                    if (STCP == CP_NONE) st64_local(own_tail, posted);
+                    else st64_agent(own_tail, posted);
                 }
                 asm volatile("" : "+v"(cw));
-                if (ask) {
-                    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(cw >> 32));
-                    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)cw);
-                    if (hi == epoch && (int32_t)lo >= need) credits_seen = lo;
+                if (role.send && (int32_t)credits_seen < need) {
+                    // A word of an earlier launch has a smaller upper half, so one
+                    // comparison covers the launch number and the count.
+                    if (__ballot(cw >= need_word) != 0ull)
+                        credits_seen = __builtin_amdgcn_readfirstlane((uint32_t)cw);
                     else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
                                          a.status))
                         give_up();
@@ -1227,16 +1233,26 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                         st128<STCP>(nxt, send_v + (uint32_t)u * W * kBlockMsg + slot_off, x);
                     }
                 }
-                ++step; ++tag; ++need;
+                ++tag; ++need;
+                need_word += 1ull;
+                asm volatile("" : "+v"(need_word));
                 g0 += a.step_blocks;
-                slot = slot + 1 == a.nslots ? 0 : slot + 1;
-                slot_off = slot ? slot_off + a.slot_bytes : 0;
+                slot_off += a.slot_bytes;
+                slot_off = slot_off == ring_bytes ? 0u : slot_off;
             };
-            while (step < whole_steps) {
+            // an odd number of steps starts with one step out of the second
+            // buffer, so that the loop is whole pairs and has one way out
+            if (whole_steps & 1u) {
+                if (role.load) fetch_step(g0, vv[1]);
+                lean_step(std::integral_constant<int, 1>{});
+            } else if (role.load) {
+                fetch_step(g0, vv[0]);
+            }
+            while (tag != end_tag) {
                 lean_step(std::integral_constant<int, 0>{});
-                if (step >= whole_steps) break;
                 lean_step(std::integral_constant<int, 1>{});
             }
+            const uint32_t step = whole_steps, slot = slot_off / a.slot_bytes;
             // what is left (a ragged or partly filled last step) starts afresh
             q.step = step; q.slot = slot; q.k0 = 0;
             q.fill(geom);
