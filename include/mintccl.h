@@ -284,6 +284,9 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
  *      and read from there, instead of into registers,
  *  16  (without 1 and 8) a streaming store of the block back into `rows`, as a
  *      copying position saves what it received (`rows` is written),
+ * 256 * k (k = 2, 4, 5, 6, 8 or 12, with 1 + 2 + 4 only) k times sixteen scalar
+ *      additions between the loads and the store of a step: the bookkeeping
+ *      of a ring step without the ring,
  * with no flags and nobody waiting for anybody.  The launch takes what the
  * device needs for that mix of accesses however well a ring schedules them:
  * the yardstick beside mint_copy_simple and mint_read_xor.  `sink` (device

@@ -155,7 +155,17 @@ __global__ void __launch_bounds__(256) step_mix_kernel(const uint8_t* __restrict
         } else if (WHAT & 1) {
             own = ll_fetch_raw(rows, 0, i * waves + wave, true, m);
         }
-        const u32x4 x = add_rn<DT_F16>(own, got);
+        u32x4 x = add_rn<DT_F16>(own, got);
+        // WHAT >> 8: that many times sixteen scalar additions between the
+        // loads and the store - the bookkeeping of a ring step without the
+        // ring (a compute unit has one scalar unit for all its wavefronts)
+        if constexpr ((WHAT >> 8) != 0) {
+            uint32_t busy = __builtin_amdgcn_readfirstlane(x.x);
+#pragma unroll
+            for (int k = 0; k < (WHAT >> 8) * 16; ++k)
+                asm volatile("s_add_u32 %0, %0, 1" : "+s"(busy) : : "scc");
+            x.x ^= busy & 0u;
+        }
         // WHAT & 16: the block also goes back to HBM, as a copying position
         // saves what it received (a streaming store of the 960 raw bytes)
         if (WHAT & 16)

@@ -526,7 +526,7 @@ int mint_read_xor(const void* src, size_t nbytes, void* out, int blocks, int thr
 
 int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t staging_bytes,
                   int waves, int iters, int what, void* sink, void* stream) {
-    if (waves <= 0 || iters <= 0 || what < 1 || what > 31 || (what & 9) == 8) return MINT_ERR_ARG;
+    if (waves <= 0 || iters <= 0 || what < 1 || (what & 9) == 8) return MINT_ERR_ARG;
     if ((what & 17) && (!rows || rows_bytes < (size_t)waves * (size_t)iters * kBlockRawLL))
         return MINT_ERR_ARG;
     if ((size_t)waves * (size_t)iters >= (1ull << 32)) return MINT_ERR_TOO_LARGE;
@@ -551,6 +551,12 @@ int mint_step_mix(const void* rows, size_t rows_bytes, void* staging, size_t sta
         case 18: kernel = step_mix_kernel<18>; break;
         case 20: kernel = step_mix_kernel<20>; break;
         case 22: kernel = step_mix_kernel<22>; break;
+        case 7 + 2 * 256: kernel = step_mix_kernel<7 + 2 * 256>; break;
+        case 7 + 4 * 256: kernel = step_mix_kernel<7 + 4 * 256>; break;
+        case 7 + 5 * 256: kernel = step_mix_kernel<7 + 5 * 256>; break;
+        case 7 + 6 * 256: kernel = step_mix_kernel<7 + 6 * 256>; break;
+        case 7 + 8 * 256: kernel = step_mix_kernel<7 + 8 * 256>; break;
+        case 7 + 12 * 256: kernel = step_mix_kernel<7 + 12 * 256>; break;
         default: return MINT_ERR_ARG;
     }
     const unsigned blocks = ((unsigned)waves + 3u) / 4u;

@@ -49,7 +49,8 @@ def step_mix(rows: torch.Tensor | None, staging: torch.Tensor | None, waves: int
     them (``what``: 1 own-row loads from ``rows``, 2 loads from ``staging``,
     4 stores into ``staging``, 8 with 1: own rows loaded straight into LDS
     instead of into registers, 16 without 1: the block is stored back into
-    ``rows``): the yardstick for what the device can do with
+    ``rows``; 256 * k with 7: k x 16 scalar additions per step between the
+    loads and the store): the yardstick for what the device can do with
     the ring kernels' mix of accesses."""
     ref = rows if rows is not None else staging
     if sink is None and not what & 20:

@@ -10,6 +10,9 @@ wavefront and step a 960-byte own-row load from HBM, a 1 KiB load from and a
                         store, next step), also with the own rows loaded
                         straight into LDS, and the mix of a copying position
                         (staging load, staging store, store to HBM);
+                        and, for the headline's 4032 wavefronts, the whole mix
+                        with 32 - 192 scalar instructions per step between
+                        the loads and the store;
 ``mint_step_mix_deep``  the loads 1, 2 or 3 steps ahead of their use and the
                         stores never waited for: 2, 3 or 4 steps in flight per
                         wavefront, each line written by one compute unit and
@@ -147,6 +150,15 @@ def main(argv: list[str]) -> int:
         ("staging load + staging store + HBM store", 22))
     for waves in waves_list:
         staging = torch.zeros(waves * 5 * 1024, dtype=torch.uint8, device=dev)
+        if not deep_only and waves == 4032:
+            # the whole mix with scalar instructions between the loads and the
+            # store of every step: what a ring step's bookkeeping may cost
+            iters = steps_for(waves, 0)
+            line = {"yardstick": "step mix and scalar instructions", "wavefronts": waves, "steps": iters}
+            for k in (0, 2, 4, 5, 6, 8, 12):
+                line[f"all three + {16 * k} scalar ms"] = round(best_ms(
+                    lambda b=7 + 256 * k: primitive.step_mix(rows, staging, waves, iters, b)), 4)
+            print(json.dumps(line), flush=True)
         if not deep_only:
             iters = steps_for(waves, 0)
             line = {"yardstick": "step mix", "steps_in_flight": 1, "wavefronts": waves,
