@@ -203,6 +203,25 @@ def test_step_mix_moves_what_it_says(dev, via_lds):
     torch.cuda.synchronize()
 
 
+def test_step_mix_with_scalar_instructions_moves_the_same(dev):
+    """what = 7 + 256 k: the scalar additions between the loads and the store
+    of a step change nothing that is stored; a k without a kernel is refused."""
+    from mintccl_amd import _lib, primitive
+    waves, iters = 29, 6
+    rows = (torch.rand(waves * iters * 480, device=dev) + 1).to(torch.float16).view(torch.uint8)
+    plain = torch.zeros(waves * 2048, dtype=torch.uint8, device=dev)
+    primitive.step_mix(rows, plain, waves, iters, what=7)
+    for k in (2, 6, 12):
+        busy = torch.zeros_like(plain)
+        primitive.step_mix(rows, busy, waves, iters, what=7 + 256 * k)
+        torch.cuda.synchronize()
+        assert torch.equal(busy, plain)
+    with pytest.raises(_lib.MintError):
+        primitive.step_mix(rows, plain, waves, iters, what=7 + 256 * 3)
+    with pytest.raises(_lib.MintError):
+        primitive.step_mix(rows, plain, waves, iters, what=5 + 256 * 2)
+
+
 def test_step_mix_saves_what_it_loads_from_staging(dev):
     """Bit 16: the block a wave took out of its staging slot goes back to HBM in
     the raw layout (lane l, l % 4 != 3: 16 bytes at vector l - l // 4; a flag
