@@ -1260,6 +1260,131 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
         }
       }
     }
+    // ---- whole steps of the Simple protocol ------------------------------------
+    // The whole group of run_group for the Simple protocol (step counter,
+    // data loads, credit, sends first, saves, fetch ahead, credit post, wait
+    // for the sends, step counter for the next rank) without the bookkeeping,
+    // as above: the general group spends 16 scalar instructions per
+    // vector-memory instruction.  All element types and roles.
+    if constexpr (PROTO == PROTO_SIMPLE && !LDSF) {
+      if (!timing && K == (uint32_t)U && ngroups) {
+        const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
+        uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
+        if (whole_steps > a.steps) whole_steps = a.steps;
+        if (whole_steps) {
+            u32x4 vv[2][U];
+            uint32_t slot_off = 0;
+            uint32_t count = 1;                              // steps done with this one
+            const uint32_t end_count = 1u + whole_steps;
+            int32_t need = 1 - (int32_t)a.nslots;
+            uint64_t need_word = flag_hi + (uint64_t)(int64_t)need;   // in vector registers, see above
+            const uint32_t recv_v = share_recv * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
+            const uint32_t send_v = share_send * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
+            const uint32_t last_full = nfull - 1u;
+            uint32_t g0 = (uint32_t)w;
+            uint64_t cw = 0;
+            // Operations between a step's sends and the wait in front of its
+            // step counter (see kOpsBehindSends): saves, fetch ahead, credit post.
+            constexpr int kBehind = (RoleT::save ? U : 0) + (RoleT::load ? U : 0) + (RoleT::recv ? 1 : 0);
+            auto fetch_step = [&](uint32_t first, u32x4 (&x)[U]) MINT_INLINE_LAMBDA {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    uint32_t g = first + (uint32_t)u * W;
+                    g = g < last_full ? g : last_full;       // beyond the whole blocks: any valid address
+                    x[u] = ld128_row(in_row + (uint64_t)g * kBlockRawSimple + m.lane * 16u);
+                }
+            };
+            auto give_up = [&]() MINT_INLINE_LAMBDA {
+                report_timeout(a.status, p, h, w, count - 1u);
+                __builtin_amdgcn_endpgm();
+            };
+            auto lean_step = [&](auto phase) MINT_INLINE_LAMBDA {
+                constexpr int B = decltype(phase)::value, B1 = B ^ 1;
+                u32x4 r[U];
+                if (role.send && (int32_t)credits_seen < need) cw = ld64_agent(nxt_tail);
+                if (role.recv) {
+                    // the sender's step counter: every line of this step is in the slot
+                    if (head_seen < count) {
+                        const uint64_t hw = ld64_agent(own_head);
+                        if (__ballot(hw >= (flag_hi | (uint64_t)count)) != 0ull)
+                            head_seen = __builtin_amdgcn_readfirstlane((uint32_t)hw);
+                        else if (!wait_count(own_head, epoch, count, head_seen, a.spin_budget, a.status))
+                            give_up();
+                    }
+                    compiler_fence();
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        r[u] = ld128<LDCP>(own, recv_v + (uint32_t)u * W * kBlockMsg, slot_off);
+                    compiler_fence();
+                }
+                asm volatile("" : "+v"(cw));
+                if (role.send && (int32_t)credits_seen < need) {
+                    if (__ballot(cw >= need_word) != 0ull)
+                        credits_seen = __builtin_amdgcn_readfirstlane((uint32_t)cw);
+                    else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
+                                         a.status))
+                        give_up();
+                }
+                u32x4 x[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    x[u] = vv[B][u];
+                    if (role.recv) {
+                        if constexpr (DT != DT_BYTES) {
+                            x[u] = role.reduce ? ll_comp<DT>(x[u], r[u]) : r[u];
+                        } else {
+                            x[u] = r[u];
+                        }
+                    }
+                    if (role.send) st128<STCP>(nxt, send_v + (uint32_t)u * W * kBlockMsg + slot_off, x[u]);
+                }
+                compiler_fence();
+                if (role.save) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        st128_row(out_row + (uint64_t)(g0 + (uint32_t)u * W) * kBlockRawSimple + m.lane * 16u, x[u]);
+                }
+                if (role.load) fetch_step(g0 + a.step_blocks, vv[B1]);
+                compiler_fence();
+                if (role.recv) {
+                    // every line of the step has been taken out of the slot (the
+                    // stores above carry what the loads returned)
+                    const uint64_t posted = flag_hi | (uint64_t)count;
+                    if (STCP == CP_NONE) st64_local(own_tail, posted);
+                    else st64_agent(own_tail, posted);
+                }
+                if (role.send) {
+                    // data first, then the step counter; what was issued behind
+                    // the sends may stay in flight
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kBehind) : "memory");
+                    const uint64_t posted = flag_hi | (uint64_t)count;
+                    if (STCP == CP_NONE) st64_local(nxt_head, posted);
+                    else st64_agent(nxt_head, posted);
+                }
+                ++count; ++need;
+                need_word += 1ull;
+                asm volatile("" : "+v"(need_word));
+                g0 += a.step_blocks;
+                slot_off += a.slot_bytes;
+                slot_off = slot_off == ring_bytes ? 0u : slot_off;
+            };
+            if (whole_steps & 1u) {
+                if (role.load) fetch_step(g0, vv[1]);
+                lean_step(std::integral_constant<int, 1>{});
+            } else if (role.load) {
+                fetch_step(g0, vv[0]);
+            }
+            while (count != end_count) {
+                lean_step(std::integral_constant<int, 0>{});
+                lean_step(std::integral_constant<int, 1>{});
+            }
+            const uint32_t step = whole_steps, slot = slot_off / a.slot_bytes;
+            q.step = step; q.slot = slot; q.k0 = 0;
+            q.fill(geom);
+            n = step;
+        }
+      }
+    }
     if constexpr (PROTO == PROTO_LL128 && DT == DT_BYTES) {
       if (!origin_done && K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
