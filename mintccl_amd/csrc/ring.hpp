@@ -1137,10 +1137,9 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // buffer instruction, the row pointer and the tag advance by constants.
     // Nothing is issued conditionally except the credit load (fetch addresses
     // are clamped into the row), so every wait leaves exactly the fetch ahead
-    // in flight.  Steps that are not whole, and a library built for wait
-    // accounting, take the general path.
+    // in flight.  Steps that are not whole take the general path.
     if constexpr (PROTO == PROTO_LL128 && DT != DT_BYTES && !LDSF) {
-      if (!timing && K == (uint32_t)U && ngroups) {
+      if (K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
         uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
         if (whole_steps > a.steps) whole_steps = a.steps;
@@ -1178,6 +1177,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 u32x4 r[U];
                 // wait_ll128 (protocol.py:161-180): asked for ahead of the polls, looked at after them
                 if (role.send && (int32_t)credits_seen < need) cw = ld64_agent(nxt_tail);
+                const uint64_t t1 = timing ? wall_clock64() : 0;
                 if (role.recv) {
                     compiler_fence();
 #pragma unroll
@@ -1198,6 +1198,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                             give_up();
                         __builtin_amdgcn_s_sleep(1);
                         compiler_fence();
+                        ++n_repoll;
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
                             if (!(pending & (1u << u))) continue;
@@ -1212,8 +1213,10 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     if (STCP == CP_NONE) st64_local(own_tail, posted);
                     else st64_agent(own_tail, posted);
                 }
+                if (timing) { t_poll += wall_clock64() - t1; ++n_groups; }
                 asm volatile("" : "+v"(cw));
                 if (role.send && (int32_t)credits_seen < need) {
+                    const uint64_t t0 = timing ? wall_clock64() : 0;
                     // A word of an earlier launch has a smaller upper half, so one
                     // comparison covers the launch number and the count.
                     if (__ballot(cw >= need_word) != 0ull)
@@ -1221,6 +1224,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
                                          a.status))
                         give_up();
+                    if (timing) t_credit += wall_clock64() - t0;
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -1267,7 +1271,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
     // as above: the general group spends 16 scalar instructions per
     // vector-memory instruction.  All element types and roles.
     if constexpr (PROTO == PROTO_SIMPLE && !LDSF) {
-      if (!timing && K == (uint32_t)U && ngroups) {
+      if (K == (uint32_t)U && ngroups) {
         const uint32_t last_idx = (uint32_t)(U - 1) * W + (uint32_t)w;
         uint32_t whole_steps = nfull > last_idx ? (nfull - 1u - last_idx) / a.step_blocks + 1u : 0u;
         if (whole_steps > a.steps) whole_steps = a.steps;
@@ -1304,6 +1308,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 if (role.send && (int32_t)credits_seen < need) cw = ld64_agent(nxt_tail);
                 if (role.recv) {
                     // the sender's step counter: every line of this step is in the slot
+                    // (its wait is booked with the credits)
+                    const uint64_t t0 = timing ? wall_clock64() : 0;
                     if (head_seen < count) {
                         const uint64_t hw = ld64_agent(own_head);
                         if (__ballot(hw >= (flag_hi | (uint64_t)count)) != 0ull)
@@ -1311,19 +1317,23 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                         else if (!wait_count(own_head, epoch, count, head_seen, a.spin_budget, a.status))
                             give_up();
                     }
+                    if (timing) t_credit += wall_clock64() - t0;
                     compiler_fence();
 #pragma unroll
                     for (int u = 0; u < U; ++u)
                         r[u] = ld128<LDCP>(own, recv_v + (uint32_t)u * W * kBlockMsg, slot_off);
                     compiler_fence();
                 }
+                if (timing) ++n_groups;
                 asm volatile("" : "+v"(cw));
                 if (role.send && (int32_t)credits_seen < need) {
+                    const uint64_t t0 = timing ? wall_clock64() : 0;
                     if (__ballot(cw >= need_word) != 0ull)
                         credits_seen = __builtin_amdgcn_readfirstlane((uint32_t)cw);
                     else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
                                          a.status))
                         give_up();
+                    if (timing) t_credit += wall_clock64() - t0;
                 }
                 u32x4 x[U];
 #pragma unroll
