@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import shutil
 import subprocess
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
@@ -132,6 +133,18 @@ def kernels_with_scratch(remarks: str) -> list[str]:
     return out
 
 
+def stores_with_scalar_offset(asm: str) -> list[str]:
+    """The 96- and 128-bit buffer stores of a device assembly listing whose
+    scalar offset operand is a register.  Such a store was seen to pick up the
+    next vector instruction's write to its first data register (the compiler
+    leaves a wait state behind a wide store only when that operand is a
+    constant), so the kernels keep a store's whole offset in the vector
+    register and build() refuses a listing that holds one."""
+    import re
+    pat = re.compile(r"^\s*buffer_store_dwordx[34]\s+v\[\d+:\d+\],\s*(?:v\d+|off),\s*s\[\d+:\d+\],\s*(s\d+|m0|vcc_lo|vcc_hi)\b")
+    return [line.strip() for line in asm.splitlines() if pat.match(line)]
+
+
 def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | None = None) -> str:
     """Compile the HIP sources for gfx950 into ``libmintccl.so`` (in-tree).
 
@@ -151,19 +164,38 @@ def build(verbose: bool = False, defines: tuple[str, ...] = (), so_path: str | N
                       os.path.join(build_dir, f"ring_family_{dt}.o")))
     procs = []
     for src, defs, obj in units:
-        cmd = ["hipcc", *HIPCC_FLAGS, *defs, "-c", "-o", obj, src]
+        # every unit compiles in a directory of its own: the compiler leaves the
+        # device assembly there (-save-temps), which is looked at below
+        tmp = obj + ".tmp"
+        shutil.rmtree(tmp, ignore_errors=True)
+        os.makedirs(tmp)
+        cmd = ["hipcc", *HIPCC_FLAGS, *defs, "-save-temps=obj", "-c", "-o",
+               os.path.join(tmp, os.path.basename(obj)), src]
         if verbose:
             print(" ".join(cmd))
-        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
-                                            text=True)))
-    errors, spilling = [], []
-    for cmd, proc in procs:
+        procs.append((cmd, tmp, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE,
+                                                      stderr=subprocess.PIPE, text=True)))
+    errors, spilling, hazards = [], [], []
+    for cmd, tmp, obj, proc in procs:
         _, err = proc.communicate()
         if proc.returncode != 0:
             errors.append(f"{' '.join(cmd)}\n{err}")
+        else:
+            listings = [f for f in os.listdir(tmp) if f.endswith("gfx950.s")]
+            if not listings:
+                errors.append(f"{' '.join(cmd)}\nleft no device assembly in {tmp}")
+            for f in listings:
+                with open(os.path.join(tmp, f)) as fh:
+                    hazards += [f"{os.path.basename(obj)}: {line}"
+                                for line in stores_with_scalar_offset(fh.read())]
+            os.replace(os.path.join(tmp, os.path.basename(obj)), obj)
+        shutil.rmtree(tmp, ignore_errors=True)
         spilling += kernels_with_scratch(err)
     if errors:
         raise RuntimeError("hipcc failed:\n" + "\n".join(errors))
+    if hazards:
+        raise RuntimeError("wide buffer stores with their offset in a scalar register "
+                           "(see stores_with_scalar_offset):\n" + "\n".join(hazards[:20]))
     if spilling:
         # A walk whose locals the optimiser could not keep in registers (it
         # happens when closures capture closures) still computes the right

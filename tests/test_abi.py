@@ -326,6 +326,24 @@ a.hpp:9:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resou
     assert "-Rpass-analysis=kernel-resource-usage" in _lib.HIPCC_FLAGS
 
 
+def test_build_refuses_wide_stores_with_a_scalar_offset_register():
+    """The build reads the device assembly: a 96- or 128-bit buffer store whose
+    scalar offset operand is a register (not the constant 0) is reported; loads
+    and narrower stores may use one."""
+    asm = """\
+\tbuffer_store_dwordx4 v[4:7], v41, s[20:23], s77 offen
+\tbuffer_store_dwordx4 v[0:3], v42, s[20:23], 0 offen
+\tbuffer_store_dwordx3 v[0:2], v42, s[20:23], s5 offen offset:16
+\tbuffer_store_dwordx2 v[0:1], v42, s[20:23], s5 offen
+\tbuffer_load_dwordx4 v[8:11], v28, s[24:27], s74 offen sc1
+\tglobal_store_dwordx4 v[2:3], v[4:7], off nt
+"""
+    bad = _lib.stores_with_scalar_offset(asm)
+    assert bad == ["buffer_store_dwordx4 v[4:7], v41, s[20:23], s77 offen",
+                   "buffer_store_dwordx3 v[0:2], v42, s[20:23], s5 offen offset:16"]
+    assert _lib.stores_with_scalar_offset("") == []
+
+
 def test_missing_library_fails_loudly(tmp_path):
     code = ("import mintccl_amd._lib as l; l.SO_PATH=%r; l._lib=None\n"
             "try:\n    l.lib()\nexcept RuntimeError as e:\n    print('RAISED', 'no CPU fallback' in str(e))\n"
