@@ -29,6 +29,7 @@
 // part in as a parent; allgather: one per row that is not its own): each has
 // a share of every slot and a credit word per wave-channel.
 #pragma once
+#include "node_step.hpp"
 #include "ring.hpp"
 
 namespace mint {
@@ -118,15 +119,50 @@ __device__ __forceinline__ void hyper_walk(const RingArgs& a, const int p, const
     const uint64_t flag_hi = (uint64_t)epoch << 32;
     uint32_t credits_seen[kHyperMaxDim] = {0u, 0u, 0u};
 
+    // The whole steps of the tuned launches (one block per wave-channel and
+    // step, XCD-local staging) run in the loop of node_step.hpp, chosen by the
+    // node's shape; what is left, and every other launch, takes the loop below.
+    uint32_t s_begin = 0;
+    if constexpr (CPI == 2) {
+        uint32_t whole = nfull > (uint32_t)w ? (nfull - 1u - (uint32_t)w) / a.step_blocks + 1u : 0u;
+        if (whole > a.steps) whole = a.steps;
+        if (K == 1u && whole && up == (DT != DT_BYTES)) {
+            NodeEdges e;
+#pragma unroll
+            for (int j = 0; j < kHyperMaxDim; ++j) {
+                e.in_off[j] = in_share[j] * a.step_msg;
+                e.out_off[j] = to_share[j] * a.step_msg;
+                e.in_tail[j] = in_tail[j];
+                e.out_tail[j] = out_tail[j];
+            }
+#define MINT_NODE(UP_, NIN_, NOUT_)                                                              \
+    if (nin == NIN_ && nout == NOUT_) {                                                          \
+        node_whole_steps<DT, CPI, UP_, NIN_, NOUT_>(a, p, h, w, whole, own, out0, out1, out2, e, \
+                                                    in_row, out_row, row_bytes, nfull,           \
+                                                    credits_seen);                               \
+        s_begin = whole;                                                                         \
+    }
+            if constexpr (DT != DT_BYTES) {
+                MINT_NODE(true, 0, 1) else MINT_NODE(true, 1, 1) else MINT_NODE(true, 2, 1)
+                else MINT_NODE(true, 1, 0) else MINT_NODE(true, 2, 0) else MINT_NODE(true, 3, 0)
+            } else {
+                MINT_NODE(false, 0, 1) else MINT_NODE(false, 0, 2) else MINT_NODE(false, 0, 3)
+                else MINT_NODE(false, 1, 0) else MINT_NODE(false, 1, 1) else MINT_NODE(false, 1, 2)
+            }
+#undef MINT_NODE
+        }
+    }
+
     // Own rows one block ahead (whole blocks only; the ragged last block of a
     // row is loaded where it is used): the load from HBM is in flight while
     // the block before it is polled for, added and sent.
     const uint32_t last_k = K - 1u;
     u32x4 ahead = {0u, 0u, 0u, 0u};
-    if (load && (uint32_t)w < nfull) ahead = ll_fetch_raw(in_row, row_bytes, (uint32_t)w, true, m);
+    if (load && s_begin == 0u && (uint32_t)w < nfull)
+        ahead = ll_fetch_raw(in_row, row_bytes, (uint32_t)w, true, m);
 
-    uint32_t slot = 0;
-    for (uint32_t s = 0; s < a.steps; ++s) {
+    uint32_t slot = s_begin % a.nslots;
+    for (uint32_t s = s_begin; s < a.steps; ++s) {
         const uint32_t tag = (epoch << 20) | (s + 1u);
         // wait_ll128 (protocol.py:161-180): the receivers have emptied the slot
         // this step goes into

@@ -26,6 +26,7 @@
 // receives from two children has two shares in each of its slots, one per
 // child, and a credit word for each.
 #pragma once
+#include "node_step.hpp"
 #include "ring.hpp"
 
 namespace mint {
@@ -172,6 +173,45 @@ __device__ __forceinline__ void tree_walk(const RingArgs& a, const int h, const 
             if (s < a.steps) {
                 const uint32_t g = s * a.step_blocks + (uint32_t)w;
                 if (g < nfull) ahead = ll_fetch_raw(in_row, row_bytes, g, true, m);
+            }
+        }
+    } else if constexpr (CPI == 2) {
+        // Every other node of a tuned launch (one block per wave-channel and
+        // step, XCD-local staging): its whole steps run in the loop of
+        // node_step.hpp, chosen by the node's shape.
+        uint32_t whole = nfull > (uint32_t)w ? (nfull - 1u - (uint32_t)w) / a.step_blocks + 1u : 0u;
+        if (whole > a.steps) whole = a.steps;
+        if (K == 1u && whole && reduce == (DT != DT_BYTES)) {
+            NodeEdges e;
+            uint32_t seen[kNodeMaxEdges] = {credits_seen[0], credits_seen[1], 0u};
+#pragma unroll
+            for (int j = 0; j < kNodeMaxEdges; ++j) {
+                const int i = j < kTreeArity ? j : 0;
+                e.in_off[j] = (uint32_t)i * a.step_msg;
+                e.out_off[j] = to_share[i] * a.step_msg;
+                e.in_tail[j] = in_tail[i];
+                e.out_tail[j] = out_tail[i];
+            }
+            bool done = false;
+#define MINT_NODE(UP_, NIN_, NOUT_)                                                               \
+    if (nin == NIN_ && nout == NOUT_) {                                                           \
+        node_whole_steps<DT, CPI, UP_, NIN_, NOUT_>(a, 0, h, w, whole, own, out0, out1, out1, e,  \
+                                                    in_row, out_row, row_bytes, nfull, seen);     \
+        done = true;                                                                              \
+    }
+            if constexpr (DT != DT_BYTES) {
+                MINT_NODE(true, 0, 1) else MINT_NODE(true, 1, 1) else MINT_NODE(true, 2, 1)
+                else MINT_NODE(true, 1, 0) else MINT_NODE(true, 2, 0)
+            } else {
+                // (the root has the loop above)
+                MINT_NODE(false, 1, 0) else MINT_NODE(false, 1, 1) else MINT_NODE(false, 1, 2)
+            }
+#undef MINT_NODE
+            if (done) {
+                credits_seen[0] = seen[0];
+                credits_seen[1] = seen[1];
+                s = whole;
+                slot = whole % a.nslots;
             }
         }
     }
