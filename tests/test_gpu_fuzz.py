@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 OPS = ["reducescatter", "allgather", "reduce", "broadcast", "allreduce"]
 
 
-def one_case(rng: random.Random, dev, case: int):
+def one_case(rng: random.Random, dev, case: int, long_rows: bool = False):
     from mintccl_amd import _lib
     from mintccl_amd.allgather import allgather
     from mintccl_amd.allreduce import allreduce
@@ -37,6 +37,8 @@ def one_case(rng: random.Random, dev, case: int):
     slot = pipes * per_pipe_blocks * 1024
     waves = pipes * rng.choice([d for d in (1, 2, 3, 4, 6, 8, 12, 16) if per_pipe_blocks % d == 0])
     n = rng.choice([1, 7, 239, 480, 481, 959, 1921, 4099, rng.randrange(1, 30000)])
+    if long_rows:
+        n = rng.randrange(60000, 400000)      # rows of many whole steps
     root = rng.randrange(world)
     shift = rng.choice([0, 0, 1, 3])
     what = f"case {case}: {op} world {world} {dt} proto {proto} place {place} cp {cp} slots {nslots}x{slot} " \
@@ -92,7 +94,7 @@ def test_random_cases_match_the_oracle(dev, seed):
     assert ran >= 60
 
 
-def one_case_of_the_other_walks(rng: random.Random, dev, case: int):
+def one_case_of_the_other_walks(rng: random.Random, dev, case: int, long_rows: bool = False):
     """Binary tree and hypercube (LL128 only): the walks beside the ring's."""
     from mintccl_amd import _lib, hypercube, tree
     from mintccl_amd.common import VirtualComm
@@ -109,6 +111,8 @@ def one_case_of_the_other_walks(rng: random.Random, dev, case: int):
     groups = world if cube else 1
     waves = groups * rng.choice([d for d in (1, 2, 3, 4, 6, 8, 12, 16) if per_share_blocks % d == 0])
     n = rng.choice([1, 7, 239, 480, 481, 959, 1921, 4099, rng.randrange(1, 30000)])
+    if long_rows:
+        n = rng.randrange(60000, 400000)      # rows of many whole steps
     root = rng.randrange(world)
     shift = rng.choice([0, 0, 1, 3])
     what = f"case {case}: {op} world {world} {dt} place {place} cp {cp} slots {nslots}x{slot} " \
@@ -156,3 +160,21 @@ def test_random_tree_and_hypercube_cases_match_the_oracle(dev, seed):
         print(what, "" if ok else "(geometry refused)", flush=True)
         ran += ok
     assert ran >= 60
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_cases_with_long_rows_match_the_oracle(dev, seed):
+    """The same walks on rows of many whole steps: the loops that run whole
+    steps (ring, Simple, tree and hypercube nodes) under random geometries."""
+    rng = random.Random(seed)
+    ran = 0
+    for case in range(24):
+        ok, what = one_case(rng, dev, seed * 1000 + case, long_rows=True)
+        print(what, "" if ok else "(geometry refused)", flush=True)
+        ran += ok
+    for case in range(12):
+        ok, what = one_case_of_the_other_walks(rng, dev, seed * 1000 + 100 + case, long_rows=True)
+        print(what, "" if ok else "(geometry refused)", flush=True)
+        ran += ok
+    assert ran >= 24
+
