@@ -12,8 +12,8 @@
 // words of the receivers are asked for ahead of the polls and looked at after
 // them; the polls of all senders go out together; the node's own row block of
 // the following step is fetched behind the polls, so that the wait for the
-// polls leaves exactly that fetch in flight (nothing is issued conditionally,
-// fetch addresses are clamped into the row); tags, credit posts, the
+// polls leaves exactly that fetch in flight (nothing behind the polls is issued
+// conditionally, fetch addresses are clamped into the row); tags, credit posts, the
 // additions, the farthest sender first, then the save or the sends.  UP: the
 // node adds what it receives to its own block (reduce, reduce-scatter); else
 // it passes on what it receives or, with no sender, its own block (broadcast,
@@ -78,9 +78,11 @@ __device__ __forceinline__ void node_whole_steps(const RingArgs& a, const int p,
     auto step = [&](auto phase) __attribute__((always_inline)) {
         constexpr int B = decltype(phase)::value, B1 = B ^ 1;
         u32x4 r[kNodeMaxEdges];
-        // wait_ll128 (protocol.py:161-180): the words of all receivers, asked for together
+        // wait_ll128 (protocol.py:161-180): the words of the receivers that have
+        // not yet been seen far enough, asked for together
 #pragma unroll
-        for (int j = 0; j < NOUT; ++j) cw[j] = ld64_agent(e.out_tail[j]);
+        for (int j = 0; j < NOUT; ++j)
+            if ((int32_t)credits_seen[j] < need) cw[j] = ld64_agent(e.out_tail[j]);
         compiler_fence();
 #pragma unroll
         for (int j = 0; j < NIN; ++j) r[j] = ld128<LDCP>(own, e.in_off[j] + lane_off, slot_off);
