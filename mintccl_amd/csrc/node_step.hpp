@@ -61,8 +61,6 @@ __device__ __forceinline__ void node_whole_steps(const RingArgs& a, const int p,
     uint32_t slot_off = 0;
     uint32_t tag = (epoch << 20) | 1u;
     int32_t need = 1 - (int32_t)a.nslots;            // credits the step needs, if positive
-    // the same as a 64-bit word, in vector registers, to compare credit words with
-    uint64_t need_word = flag_hi + (uint64_t)(int64_t)need;
     uint32_t g0 = (uint32_t)w;
     u32x4 vv[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
     uint64_t cw[kNodeMaxEdges] = {0, 0, 0};
@@ -116,8 +114,8 @@ __device__ __forceinline__ void node_whole_steps(const RingArgs& a, const int p,
         for (int j = 0; j < NOUT; ++j) {
             asm volatile("" : "+v"(cw[j]));
             if ((int32_t)credits_seen[j] < need) {
-                // (a word of an earlier launch has a smaller upper half)
-                if (__ballot(cw[j] >= need_word) != 0ull)
+                // (compared in vector registers: every lane holds the word)
+                if (__ballot((uint32_t)(cw[j] >> 32) == epoch && (int32_t)(uint32_t)cw[j] >= need) != 0ull)
                     credits_seen[j] = __builtin_amdgcn_readfirstlane((uint32_t)cw[j]);
                 else if (!wait_count(e.out_tail[j], epoch, (uint32_t)need, credits_seen[j],
                                      a.spin_budget, a.status))
@@ -144,8 +142,6 @@ __device__ __forceinline__ void node_whole_steps(const RingArgs& a, const int p,
             if (NOUT > 2) st128<STCP>(out2, e.out_off[2] + at, x);
         }
         ++tag; ++need;
-        need_word += 1ull;
-        asm volatile("" : "+v"(need_word));
         g0 += a.step_blocks;
         slot_off += a.slot_bytes;
         slot_off = slot_off == ring_bytes ? 0u : slot_off;

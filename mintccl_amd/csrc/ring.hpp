@@ -1151,9 +1151,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             uint32_t tag = (epoch << 20) | 1u;
             const uint32_t end_tag = tag + whole_steps;
             int32_t need = 1 - (int32_t)a.nslots;
-            // the same as a 64-bit word to compare the credit word with, kept in
-            // vector registers (a CU has one scalar unit and sixty-four vector lanes)
-            uint64_t need_word = flag_hi + (uint64_t)(int64_t)need;
             const uint32_t recv_v = share_recv * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t send_v = share_send * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t last_full = nfull - 1u;
@@ -1221,9 +1218,8 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 asm volatile("" : "+v"(cw));
                 if (role.send && (int32_t)credits_seen < need) {
                     const uint64_t t0 = timing ? wall_clock64() : 0;
-                    // A word of an earlier launch has a smaller upper half, so one
-                    // comparison covers the launch number and the count.
-                    if (__ballot(cw >= need_word) != 0ull)
+                    // (compared in vector registers: every lane holds the word)
+                    if (__ballot((uint32_t)(cw >> 32) == epoch && (int32_t)(uint32_t)cw >= need) != 0ull)
                         credits_seen = __builtin_amdgcn_readfirstlane((uint32_t)cw);
                     else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
                                          a.status))
@@ -1243,8 +1239,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 }
                 if (role.recv) __builtin_amdgcn_s_setprio(0);
                 ++tag; ++need;
-                need_word += 1ull;
-                asm volatile("" : "+v"(need_word));
                 g0 += a.step_blocks;
                 slot_off += a.slot_bytes;
                 slot_off = slot_off == ring_bytes ? 0u : slot_off;
@@ -1286,7 +1280,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
             uint32_t count = 1;                              // steps done with this one
             const uint32_t end_count = 1u + whole_steps;
             int32_t need = 1 - (int32_t)a.nslots;
-            uint64_t need_word = flag_hi + (uint64_t)(int64_t)need;   // in vector registers, see above
             const uint32_t recv_v = share_recv * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t send_v = share_send * a.step_msg + (uint32_t)w * kBlockMsg + m.lane * 16u;
             const uint32_t last_full = nfull - 1u;
@@ -1317,7 +1310,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     const uint64_t t0 = timing ? wall_clock64() : 0;
                     if (head_seen < count) {
                         const uint64_t hw = ld64_agent(own_head);
-                        if (__ballot(hw >= (flag_hi | (uint64_t)count)) != 0ull)
+                        if (__ballot((uint32_t)(hw >> 32) == epoch && (uint32_t)hw >= count) != 0ull)
                             head_seen = __builtin_amdgcn_readfirstlane((uint32_t)hw);
                         else if (!wait_count(own_head, epoch, count, head_seen, a.spin_budget, a.status))
                             give_up();
@@ -1333,7 +1326,7 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                 asm volatile("" : "+v"(cw));
                 if (role.send && (int32_t)credits_seen < need) {
                     const uint64_t t0 = timing ? wall_clock64() : 0;
-                    if (__ballot(cw >= need_word) != 0ull)
+                    if (__ballot((uint32_t)(cw >> 32) == epoch && (int32_t)(uint32_t)cw >= need) != 0ull)
                         credits_seen = __builtin_amdgcn_readfirstlane((uint32_t)cw);
                     else if (!wait_count(nxt_tail, epoch, (uint32_t)need, credits_seen, a.spin_budget,
                                          a.status))
@@ -1377,8 +1370,6 @@ __device__ __forceinline__ void ring_walk(const RingArgs& a, const int p, const 
                     else st64_agent(nxt_head, posted);
                 }
                 ++count; ++need;
-                need_word += 1ull;
-                asm volatile("" : "+v"(need_word));
                 g0 += a.step_blocks;
                 slot_off += a.slot_bytes;
                 slot_off = slot_off == ring_bytes ? 0u : slot_off;

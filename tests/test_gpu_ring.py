@@ -947,3 +947,20 @@ def test_rows_beyond_4_gib(dev):
     run_broadcast(comm, bufs, 0)
     for b in bufs[1:]:
         assert torch.equal(b, src)
+
+
+@pytest.mark.parametrize("proto", [0, 1])
+def test_a_smaller_epoch_after_a_larger_one_on_the_same_staging(dev, proto):
+    """The epoch of a launch only has to differ from the earlier ones on the
+    same staging, not to exceed them: credit words and step counters left by a
+    launch with a larger epoch must not pass for this launch's (rows of many
+    steps through three slots, so every sender has to wait for credits)."""
+    world, n = 8, 200000
+    comm = make_comm(world, protocol=proto, buff_size_=3 * 8 * 16 * 1024, nslots=3, waves_per_rank=8 * 16)
+    for epoch_before in (900, 40):
+        host = rank_rows(world, n, "f16", seed0=5000 + epoch_before)
+        bufs = [h.to(dev) for h in host]
+        comm.epoch = epoch_before          # the launch takes the next one
+        run_reducescatter(comm, bufs)
+        assert same(bufs, ring.reducescatter([as_bytes(h) for h in host], "f16"))
+
